@@ -1,0 +1,139 @@
+/*
+ * vt_oracle.h - CPU restatement of the voxtral-tts.c backbone / acoustic hot path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This library is the checker that the HIP path is
+ * compared against (tests, the smoke check, and the cpu_baseline leg of the
+ * benchmark).  Nothing in the product library links, loads or calls it.
+ *
+ * Every function restates, in plain sequential IEEE fp32 with no FMA
+ * contraction, the arithmetic of a function of the reference CPU path; the
+ * reference file:line it follows is cited at each definition in vt_oracle.c.
+ *
+ * Pin status (what fixes each function besides this restatement):
+ *   - all functions: bit-identical to the compiled reference sources
+ *     (oracle/_ref, built from /root/reference by oracle/Makefile) in
+ *     tests/test_oracle_vs_ref.py, and frozen in tests/golden/ fixtures
+ *     produced by that compiled reference.
+ *   - orc_linear_bf16 with seq_len > 1 follows the reference's no-BLAS
+ *     triple loop (voxtral_tts_kernels.c:127-138).  The reference's BLAS
+ *     build delegates the summation order to an unpinned third-party
+ *     cblas_sgemm, and no reference test fixes results there: for
+ *     seq_len > 1 parity with a BLAS build of the reference is
+ *     "parity unpinned"; parity with the no-BLAS build is pinned.
+ */
+#ifndef VT_ORACLE_H
+#define VT_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Model dimensions (voxtral_tts.h:19-44, 65-79). */
+#define ORC_DIM        3072
+#define ORC_HEADS      32
+#define ORC_KV_HEADS   8
+#define ORC_HEAD_DIM   128
+#define ORC_Q_DIM      (ORC_HEADS * ORC_HEAD_DIM)     /* 4096 */
+#define ORC_KV_DIM     (ORC_KV_HEADS * ORC_HEAD_DIM)  /* 1024 */
+#define ORC_FFN        9216
+#define ORC_EPS        1e-5f
+#define ORC_ROPE_THETA 1000000.0f
+#define ORC_ACOUSTIC_DIM 36
+#define ORC_FLOW_STEPS 8
+#define ORC_CFG_ALPHA  1.2f
+#define ORC_FSQ_LEVELS 21
+#define ORC_SEM_PADDED 8320
+#define ORC_SEM_SIZE   8192
+#define ORC_CODES_PER_FRAME 37
+
+/* One transformer layer's weights (field meaning as voxtral_tts.h:101-114). */
+typedef struct {
+    const uint16_t *wq, *wk, *wv, *wo;   /* bf16 [4096,3072] [1024,3072] [1024,3072] [3072,4096] */
+    const float *attention_norm;         /* f32 [3072] */
+    const uint16_t *w1, *w2, *w3;        /* bf16 [9216,3072] [3072,9216] [9216,3072] */
+    const float *ffn_norm;               /* f32 [3072] */
+} orc_layer_t;
+
+/* Acoustic transformer weights (voxtral_tts.h:146-165). */
+typedef struct {
+    const float *time_inv_freq;          /* f32 [1536] */
+    const uint16_t *input_proj;          /* bf16 [3072,36] */
+    const uint16_t *time_proj;           /* bf16 [3072,3072] */
+    const uint16_t *llm_proj;            /* bf16 [3072,3072] */
+    const uint16_t *semantic_out;        /* bf16 [8320,3072] */
+    const float *semantic_out_bias;      /* f32 [8320] or NULL */
+    const uint16_t *acoustic_out;        /* bf16 [36,3072] */
+    const float *norm;                   /* f32 [3072] */
+    const orc_layer_t *layers;           /* n_layers entries */
+    int n_layers;
+} orc_acoustic_t;
+
+/* Row-parallel worker count for the matvec / linear / attention loops.
+ * Rows (and heads) are independent, so results are bit-identical for any
+ * count; the reference itself is single-threaded (count 1, the default). */
+void orc_set_threads(int n);
+int  orc_get_threads(void);
+
+/* Elementwise + bf16 helpers */
+void orc_add_inplace(float *a, const float *b, int n);
+void orc_mul_inplace(float *a, const float *b, int n);
+void orc_silu(float *x, int n);
+void orc_bf16_to_f32_buf(float *dst, const uint16_t *src, size_t n);
+void orc_embed_token_bf16(float *out, const uint16_t *emb, int token_id, int dim);
+
+/* y[s,o] = bias[o]? + sum_k W[o,k]*x[s,k], k ascending, fp32 */
+void orc_linear_bf16(float *y, const float *x, const uint16_t *W_bf16,
+                     const float *bias, int seq_len, int in_dim, int out_dim);
+
+void orc_rms_norm(float *out, const float *x, const float *weight,
+                  int seq_len, int hidden, float eps);
+void orc_compute_rope_freqs(float *freqs, const int *pos, int seq, int dim, float theta);
+void orc_apply_rope(float *x, const float *freqs, int seq, int heads, int head_dim);
+
+void orc_causal_attention(float *out, const float *Q, const float *K, const float *V,
+                          int seq_q, int seq_k, int n_heads, int n_kv_heads,
+                          int head_dim, float scale, int window_size, int q_offset);
+void orc_bidirectional_attention(float *out, const float *Q, const float *K, const float *V,
+                                 int seq_len, int n_heads, int n_kv_heads,
+                                 int head_dim, float scale);
+
+/* RNG */
+void  orc_rng_seed(uint64_t *state, uint64_t seed);
+float orc_randn(uint64_t *state);
+void  orc_randn_fill(uint64_t *state, float *buf, int n);
+
+/* Backbone: one decode step at position pos.  KV caches are
+ * f32 [n_layers, kv_max, 1024]; row pos of every layer is written. */
+void orc_llm_forward(const orc_layer_t *layers, int n_layers, const float *final_norm,
+                     float *kv_k, float *kv_v, int kv_max, int pos,
+                     const float *input_embed, float *out_hidden);
+
+/* Backbone prefill of seq_len rows starting at start_pos.  If out_x is not
+ * NULL it receives the [seq_len,3072] residual stream after the last layer
+ * (before the final norm), which the reference computes and discards. */
+void orc_llm_prefill(const orc_layer_t *layers, int n_layers,
+                     float *kv_k, float *kv_v, int kv_max, int start_pos,
+                     const float *embeds, int seq_len, float *out_x);
+
+/* Acoustic transformer */
+void orc_time_embedding(const float *inv_freq, float t_val, float *out, int dim);
+void orc_default_time_inv_freq(float *inv_freq, int half_dim);
+void orc_predict_velocity(const orc_acoustic_t *ac, const float *x_t,
+                          const float *llm_hidden, float t_val, float *out_velocity);
+/* One audio frame: semantic argmax, noise, 7 Euler steps with CFG, FSQ.
+ * out_x (optional, 36 floats) receives the final latent before quantisation. */
+void orc_acoustic_forward(const orc_acoustic_t *ac, const float *llm_hidden,
+                          uint64_t *rng_state, int *out_codes, float *out_x);
+
+/* Audio-code embedding sum feeding the next backbone step
+ * (37 rows of a bf16 table, offsets = cumulative unpadded codebook sizes). */
+void orc_audio_embed_forward(const uint16_t *emb_bf16, const int *offsets,
+                             const int *codes, float *out_embed, int dim);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VT_ORACLE_H */
