@@ -1,0 +1,208 @@
+/*
+ * voxtral_tts_hip.h - C ABI of the MI355X (gfx950) backend for the
+ * voxtral-tts.c LLM-backbone / acoustic-transformer hot path.
+ *
+ * The entry points mirror, one for one, the GPU backend interface of the
+ * reference (voxtral_tts_cuda.h:89-185): same argument order and meaning,
+ * same host-pointer / device-pointer conventions, same `int` 0 / -1 results
+ * for init and uploads and `void` compute entry points.  The reference
+ * declaration each one replaces is cited at its prototype.  Entry points with
+ * no counterpart in the reference are grouped at the end and say so.
+ *
+ * Plain C, no HIP or torch types in any signature: device memory is passed as
+ * `void *` / `float *` addresses obtained from tts_hip_alloc (or from any
+ * other allocator of the same HIP device).
+ *
+ * One global context, not thread-safe, one internal stream; every entry
+ * point that takes host pointers is synchronous, every entry point that
+ * takes device pointers is asynchronous on the internal stream (call
+ * tts_hip_sync) - the conventions of the reference backend.
+ */
+#ifndef VOXTRAL_TTS_HIP_H
+#define VOXTRAL_TTS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TTS_HIP_DEC_LAYERS 26
+#define TTS_HIP_AC_LAYERS  3
+
+/* ---- host-side weight structs consumed through `void *` -------------------
+ * Field order and types are the upload ABI: they equal tts_dec_layer_t /
+ * tts_decoder_t (voxtral_tts.h:101-125) and tts_ac_layer_t / tts_acoustic_t
+ * (voxtral_tts.h:131-165), so a pointer to the reference's structs can be
+ * passed unchanged. */
+typedef struct {
+    uint16_t *wq_bf16;        /* [4096, 3072] */
+    uint16_t *wk_bf16;        /* [1024, 3072] */
+    uint16_t *wv_bf16;        /* [1024, 3072] */
+    uint16_t *wo_bf16;        /* [3072, 4096] */
+    float *attention_norm;    /* [3072] */
+    uint16_t *w1_bf16;        /* [9216, 3072] gate */
+    uint16_t *w2_bf16;        /* [3072, 9216] down */
+    uint16_t *w3_bf16;        /* [9216, 3072] up */
+    float *ffn_norm;          /* [3072] */
+} tts_hip_host_layer_t;
+
+typedef struct {
+    uint16_t *tok_embeddings_bf16;                    /* [131072, 3072] or NULL */
+    tts_hip_host_layer_t layers[TTS_HIP_DEC_LAYERS];
+    float *norm;                                      /* [3072] */
+} tts_hip_host_decoder_t;
+
+typedef struct {
+    float *time_inv_freq;              /* [1536] */
+    uint16_t *input_proj_bf16;         /* [3072, 36] */
+    uint16_t *time_proj_bf16;          /* [3072, 3072] */
+    uint16_t *llm_proj_bf16;           /* [3072, 3072] */
+    uint16_t *semantic_out_bf16;       /* [8320, 3072] */
+    float *semantic_out_bias;          /* [8320] or NULL */
+    uint16_t *acoustic_out_bf16;       /* [36, 3072] */
+    float *norm;                       /* [3072] */
+    tts_hip_host_layer_t layers[TTS_HIP_AC_LAYERS];
+} tts_hip_host_acoustic_t;
+
+/* ---- exported context (replaces the fields of `g_cuda` that code outside the
+ * backend touches: voxtral_tts_cuda.h:51-54,78 read at voxtral_tts_llm.c:380-381) */
+typedef struct {
+    float *kv_cache_k_gpu;    /* f32 [26, kv_cache_max, 1024] */
+    float *kv_cache_v_gpu;
+    int kv_cache_max;
+    int initialized;
+    int n_cu;                 /* compute units of the device */
+    int dec_layers_uploaded;
+    int ac_layers_uploaded;
+} tts_hip_ctx_t;
+
+extern tts_hip_ctx_t g_hip;
+
+/* ---- init / upload / teardown -------------------------------------------- */
+
+/* replaces tts_cuda_init (voxtral_tts_cuda.h:89). Idempotent. 0 / -1. */
+int tts_hip_init(int kv_cache_max);
+/* replaces tts_cuda_upload_llm_weights (voxtral_tts_cuda.h:92); decoder_ptr is a
+ * tts_decoder_t * / tts_hip_host_decoder_t *.  Copies; the host keeps ownership. */
+int tts_hip_upload_llm_weights(void *decoder_ptr);
+/* replaces tts_cuda_upload_acoustic_weights (voxtral_tts_cuda.h:93). */
+int tts_hip_upload_acoustic_weights(void *acoustic_ptr);
+/* replaces tts_cuda_free (voxtral_tts_cuda.h:96). */
+void tts_hip_free(void);
+/* replaces tts_cuda_available (voxtral_tts_cuda.h:99). */
+int tts_hip_available(void);
+
+/* ---- linear ---------------------------------------------------------------- */
+
+/* replaces tts_cuda_linear_bf16 (voxtral_tts_cuda.h:109-111): y = x W^T, x and y
+ * each host or device, W_gpu device bf16 [out_dim, in_dim]; W_gpu == NULL
+ * uploads W_bf16 from the host for the call. */
+void tts_hip_linear_bf16(float *y, const float *x, const uint16_t *W_bf16,
+                         int seq_len, int in_dim, int out_dim, const void *W_gpu);
+
+/* ---- kernel-level operators on device pointers ---------------------------- */
+
+/* replaces tts_cuda_rms_norm (voxtral_tts_cuda.h:118-119) */
+void tts_hip_rms_norm(float *d_out, const float *d_x, const float *d_weight,
+                      int seq_len, int dim, float eps);
+/* replaces tts_cuda_apply_rope (voxtral_tts_cuda.h:122-123); d_freqs is
+ * f32 [seq, head_dim/2, 2] (cos, sin) and IS honoured (the reference ignores it). */
+void tts_hip_apply_rope(float *d_x, const float *d_freqs, int seq, int heads, int head_dim);
+/* replaces tts_cuda_compute_rope_freqs (voxtral_tts_cuda.h:126-127), a stub in
+ * the reference; here it fills d_freqs for positions start_pos..start_pos+seq-1. */
+void tts_hip_compute_rope_freqs(float *d_freqs, int start_pos, int seq, int dim, float theta);
+/* replaces tts_cuda_silu_mul (voxtral_tts_cuda.h:130) */
+void tts_hip_silu_mul(float *d_gate, const float *d_up, int n);
+/* replaces tts_cuda_add_inplace (voxtral_tts_cuda.h:133) */
+void tts_hip_add_inplace(float *d_a, const float *d_b, int n);
+/* replaces tts_cuda_causal_attention_decode (voxtral_tts_cuda.h:136-139);
+ * kv_cache_stride is the row stride in floats (0 = n_kv_heads*head_dim). */
+void tts_hip_causal_attention_decode(float *d_out, const float *d_Q, const float *d_K_cache,
+                                     const float *d_V_cache, int seq_k, int n_heads,
+                                     int n_kv_heads, int head_dim, float scale,
+                                     int kv_cache_stride);
+/* replaces tts_cuda_causal_attention_prefill (voxtral_tts_cuda.h:142-145) */
+void tts_hip_causal_attention_prefill(float *d_out, const float *d_Q, const float *d_K,
+                                      const float *d_V, int seq_len, int start_pos,
+                                      int n_heads, int n_kv_heads, int head_dim, float scale);
+/* replaces tts_cuda_bidirectional_attention (voxtral_tts_cuda.h:148-150) */
+void tts_hip_bidirectional_attention(float *d_out, const float *d_Q, const float *d_K,
+                                     const float *d_V, int seq_len, int n_heads,
+                                     int n_kv_heads, int head_dim, float scale);
+/* replaces tts_cuda_embed_token (voxtral_tts_cuda.h:153-154) */
+void tts_hip_embed_token(float *d_out, const void *d_embeddings_bf16, int token_id, int dim);
+
+/* ---- backbone --------------------------------------------------------------- */
+
+/* replaces tts_cuda_llm_forward (voxtral_tts_cuda.h:161-162): one decode step
+ * at cache position pos; host pointers; synchronous. */
+void tts_hip_llm_forward(float *out_hidden, const float *input_embed, int pos);
+/* replaces tts_cuda_llm_prefill (voxtral_tts_cuda.h:165): fills cache rows
+ * start_pos..start_pos+seq_len-1 on the device; host pointer; synchronous. */
+void tts_hip_llm_prefill(const float *embeds, int seq_len, int start_pos);
+
+/* ---- acoustic transformer -------------------------------------------------- */
+
+/* replaces tts_cuda_predict_velocity (voxtral_tts_cuda.h:172-174) */
+void tts_hip_predict_velocity(float *out_velocity, const float *x_t,
+                              const float *llm_hidden, float t_val);
+
+/* ---- transfers --------------------------------------------------------------- */
+
+/* replace tts_cuda_to_device / to_host / memset / alloc / free_ptr / sync
+ * (voxtral_tts_cuda.h:180-185) */
+void tts_hip_to_device(void *d_dst, const void *h_src, size_t bytes);
+void tts_hip_to_host(void *h_dst, const void *d_src, size_t bytes);
+void tts_hip_memset(void *d_ptr, int value, size_t bytes);
+void *tts_hip_alloc(size_t bytes);
+void tts_hip_free_ptr(void *d_ptr);
+void tts_hip_sync(void);
+
+/* ==== entry points with no counterpart in the reference ===================== */
+
+/* Upload only the first n_layers decoder layers (1..26); used for one-layer
+ * and few-layer configurations.  Sources may be host or device pointers. */
+int tts_hip_upload_llm_weights_n(void *decoder_ptr, int n_layers);
+/* Upload one decoder layer (index 0..25) from host or device pointers. */
+int tts_hip_upload_llm_layer(int layer, const tts_hip_host_layer_t *src);
+/* Final-norm weights f32 [3072], host or device pointer. */
+int tts_hip_upload_llm_norm(const float *norm);
+
+/* One decode step on device-resident buffers, asynchronous on the internal
+ * stream: d_input_embed f32 [3072] -> d_out_hidden f32 [3072]. */
+void tts_hip_llm_forward_device(float *d_out_hidden, const float *d_input_embed, int pos);
+/* One decoder layer at batch 1 on a device-resident hidden state (in place),
+ * appending row pos of that layer's cache.  Asynchronous. */
+void tts_hip_layer_decode(int layer, float *d_hidden, int pos);
+/* Prefill that also returns the residual stream after the last layer
+ * ([seq_len, 3072], host pointer, may be NULL). */
+void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int start_pos, float *out_x);
+
+/* Conditional + unconditional velocity in one batch-2 pass (classifier-free
+ * guidance): equals predict_velocity(x_t, llm_hidden, t) and
+ * predict_velocity(x_t, 0, t) (voxtral_tts_acoustic.c:345-348). */
+void tts_hip_predict_velocity_cfg(float *out_v_cond, float *out_v_uncond, const float *x_t,
+                                  const float *llm_hidden, float t_val);
+/* One audio frame on the device: semantic head + argmax, 7 Euler steps with
+ * CFG from the caller's noise x0[36], FSQ quantisation -> codes[37]
+ * (voxtral_tts_acoustic.c:268-373).  Host pointers; synchronous.  out_x
+ * (optional) receives the final latent. */
+void tts_hip_acoustic_frame(int *out_codes, const float *llm_hidden, const float *x0,
+                            float *out_x);
+
+/* 0 = persistent whole-step kernel (default), 1 = one kernel per phase. */
+void tts_hip_set_decode_mode(int mode);
+/* Number of failed calls since init, and the text of the last failure. */
+int tts_hip_error_count(void);
+const char *tts_hip_last_error(void);
+
+/* Event timing on the internal stream (for benchmarks). */
+void tts_hip_timer_start(void);
+float tts_hip_timer_stop_ms(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VOXTRAL_TTS_HIP_H */

@@ -1,0 +1,142 @@
+"""Host-side Python mirror of the C ABI in include/voxtral_tts_hip.h.
+
+The product is the shared library csrc/libvoxtral_tts_hip.so (hand-written HIP
+for gfx950 behind `extern "C"` entry points named after the reference's
+`tts_cuda_*` interface).  This module only loads it with ctypes and declares
+the signatures; there is no CPU fallback: a missing library raises.
+
+The directory name is not a Python identifier; load it with
+`importlib` (see `load()` in tests/hipsupport.py or __graft_entry__.py).
+"""
+import ctypes as C
+import os
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_PATH = os.path.join(CSRC, "libvoxtral_tts_hip.so")
+
+DEC_LAYERS = 26
+AC_LAYERS = 3
+
+f32p = C.POINTER(C.c_float)
+u16p = C.POINTER(C.c_uint16)
+i32p = C.POINTER(C.c_int)
+vp = C.c_void_p
+
+
+class HostLayer(C.Structure):
+    """tts_hip_host_layer_t == tts_dec_layer_t / tts_ac_layer_t (voxtral_tts.h:101-114)."""
+    _fields_ = [("wq_bf16", vp), ("wk_bf16", vp), ("wv_bf16", vp), ("wo_bf16", vp),
+                ("attention_norm", vp),
+                ("w1_bf16", vp), ("w2_bf16", vp), ("w3_bf16", vp),
+                ("ffn_norm", vp)]
+
+
+class HostDecoder(C.Structure):
+    """tts_hip_host_decoder_t == tts_decoder_t (voxtral_tts.h:116-125)."""
+    _fields_ = [("tok_embeddings_bf16", vp), ("layers", HostLayer * DEC_LAYERS), ("norm", vp)]
+
+
+class HostAcoustic(C.Structure):
+    """tts_hip_host_acoustic_t == tts_acoustic_t (voxtral_tts.h:146-165)."""
+    _fields_ = [("time_inv_freq", vp), ("input_proj_bf16", vp), ("time_proj_bf16", vp),
+                ("llm_proj_bf16", vp), ("semantic_out_bf16", vp), ("semantic_out_bias", vp),
+                ("acoustic_out_bf16", vp), ("norm", vp), ("layers", HostLayer * AC_LAYERS)]
+
+
+class HipCtx(C.Structure):
+    """tts_hip_ctx_t (the exported global g_hip)."""
+    _fields_ = [("kv_cache_k_gpu", vp), ("kv_cache_v_gpu", vp), ("kv_cache_max", C.c_int),
+                ("initialized", C.c_int), ("n_cu", C.c_int), ("dec_layers_uploaded", C.c_int),
+                ("ac_layers_uploaded", C.c_int)]
+
+
+# name -> (restype, argtypes); every symbol include/voxtral_tts_hip.h declares
+SIGNATURES = {
+    "tts_hip_init": (C.c_int, [C.c_int]),
+    "tts_hip_upload_llm_weights": (C.c_int, [vp]),
+    "tts_hip_upload_acoustic_weights": (C.c_int, [vp]),
+    "tts_hip_free": (None, []),
+    "tts_hip_available": (C.c_int, []),
+    "tts_hip_linear_bf16": (None, [vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
+    "tts_hip_rms_norm": (None, [vp, vp, vp, C.c_int, C.c_int, C.c_float]),
+    "tts_hip_apply_rope": (None, [vp, vp, C.c_int, C.c_int, C.c_int]),
+    "tts_hip_compute_rope_freqs": (None, [vp, C.c_int, C.c_int, C.c_int, C.c_float]),
+    "tts_hip_silu_mul": (None, [vp, vp, C.c_int]),
+    "tts_hip_add_inplace": (None, [vp, vp, C.c_int]),
+    "tts_hip_causal_attention_decode": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int,
+                                               C.c_float, C.c_int]),
+    "tts_hip_causal_attention_prefill": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int,
+                                                C.c_int, C.c_float]),
+    "tts_hip_bidirectional_attention": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int,
+                                               C.c_float]),
+    "tts_hip_embed_token": (None, [vp, vp, C.c_int, C.c_int]),
+    "tts_hip_llm_forward": (None, [vp, vp, C.c_int]),
+    "tts_hip_llm_prefill": (None, [vp, C.c_int, C.c_int]),
+    "tts_hip_predict_velocity": (None, [vp, vp, vp, C.c_float]),
+    "tts_hip_to_device": (None, [vp, vp, C.c_size_t]),
+    "tts_hip_to_host": (None, [vp, vp, C.c_size_t]),
+    "tts_hip_memset": (None, [vp, C.c_int, C.c_size_t]),
+    "tts_hip_alloc": (vp, [C.c_size_t]),
+    "tts_hip_free_ptr": (None, [vp]),
+    "tts_hip_sync": (None, []),
+    "tts_hip_upload_llm_weights_n": (C.c_int, [vp, C.c_int]),
+    "tts_hip_upload_llm_layer": (C.c_int, [C.c_int, C.POINTER(HostLayer)]),
+    "tts_hip_upload_llm_norm": (C.c_int, [vp]),
+    "tts_hip_llm_forward_device": (None, [vp, vp, C.c_int]),
+    "tts_hip_layer_decode": (None, [C.c_int, vp, C.c_int]),
+    "tts_hip_llm_prefill_out": (None, [vp, C.c_int, C.c_int, vp]),
+    "tts_hip_predict_velocity_cfg": (None, [vp, vp, vp, vp, C.c_float]),
+    "tts_hip_acoustic_frame": (None, [vp, vp, vp, vp]),
+    "tts_hip_set_decode_mode": (None, [C.c_int]),
+    "tts_hip_error_count": (C.c_int, []),
+    "tts_hip_last_error": (C.c_char_p, []),
+    "tts_hip_timer_start": (None, []),
+    "tts_hip_timer_stop_ms": (C.c_float, []),
+}
+
+_lib = None
+
+
+def build(force=False):
+    """Compile the library for gfx950 with hipcc (cross-compiles without a GPU)."""
+    if force:
+        subprocess.check_call(["make", "-s", "-C", CSRC, "clean"])
+    subprocess.check_call(["make", "-s", "-j8", "-C", CSRC])
+    return LIB_PATH
+
+
+def lib():
+    """The loaded C-ABI library with typed entry points.  Fails loudly if it
+    has not been built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is not built; run `make -C {CSRC}` "
+                               "(or __graft_entry__.build())")
+        l = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(l, name)          # AttributeError if the symbol is missing
+            fn.restype = res
+            fn.argtypes = args
+        _lib = l
+    return _lib
+
+
+def ctx():
+    """The exported global context g_hip."""
+    return HipCtx.in_dll(lib(), "g_hip")
+
+
+class HipError(RuntimeError):
+    pass
+
+
+def check_errors(before):
+    """Raise if the library recorded a failure since `before` (compute entry
+    points are `void`, like the reference's)."""
+    l = lib()
+    n = l.tts_hip_error_count()
+    if n != before:
+        raise HipError(l.tts_hip_last_error().decode())

@@ -1,0 +1,402 @@
+/*
+ * vt_decode_phases.h - the five phases of one decoder layer at batch 1, as
+ * device functions shared by the per-phase kernels and by the persistent
+ * whole-step kernel.
+ *
+ * Every GEMV phase streams bf16 weight rows with 16-byte non-temporal loads:
+ * a wave owns whole rows (or a fixed k-range of rows), each lane keeps its
+ * slice of the activation vector in registers (lane l holds elements
+ * c*512 + l*8 .. +8 of every 512-element chunk c), products are accumulated
+ * with fp32 FMA per lane and summed across the wave in a fixed DPP order.
+ * Rows are kept in a ring of D row buffers, so D rows of loads are in flight
+ * per wave; the first D rows of a phase can be requested before the grid
+ * barrier that precedes the phase (weights do not depend on activations).
+ *
+ * Operation order follows the reference CPU decode step
+ * (voxtral_tts_llm.c:205-264): RMSNorm -> q,k,v -> RoPE -> cache append ->
+ * attention -> wo + residual -> RMSNorm -> w1,w3 -> SiLU*up -> w2 + residual.
+ */
+#ifndef VT_DECODE_PHASES_H
+#define VT_DECODE_PHASES_H
+
+#include "vt_device.h"
+
+#define VT_RING 18            /* 16-byte buffers per lane in the row ring */
+#define VT_ATT_STRIDE 132     /* floats per attention partial: m, l, pad, pad, o[128] */
+
+/* Device-side weights of one layer, laid out at upload:
+ *   wqkv = [wq ; wk ; wv]            [6144, 3072]
+ *   w13  = rows interleaved (w1 row j, w3 row j)   [18432, 3072]     */
+struct vt_layer_dev {
+    const uint16_t *wqkv;
+    const uint16_t *wo;
+    const uint16_t *w13;
+    const uint16_t *w2;
+    const float *attn_norm;
+    const float *ffn_norm;
+};
+
+struct vt_step_args {
+    const vt_layer_dev *layers;
+    int n_layers;
+    int first_layer;              /* global index of layers[0] in the KV cache */
+    const float *final_norm;      /* NULL: skip the final RMSNorm */
+    float *kv_k, *kv_v;           /* f32 [layers, kv_max, 1024] */
+    int kv_max;
+    int pos;
+    const float *rope;            /* f32 [kv_max, 64, 2] (cos, sin) */
+    const float *in_embed;        /* f32 [3072] */
+    float *out_hidden;            /* f32 [3072] */
+    float *x;                     /* residual stream */
+    float *q, *attn, *h;          /* [4096], [4096], [9216] */
+    float *att_part;              /* [32 heads, n_chunks, VT_ATT_STRIDE] */
+    unsigned int *att_cnt;        /* [n_layers * 8], zero at phase start */
+};
+
+/* ---- activation slices ---------------------------------------------------- */
+
+template <int NK>
+__device__ __forceinline__ void vt_load_slice(f32x4 (&xa)[NK], f32x4 (&xb)[NK],
+                                              const float *x, int kofs) {
+    const int lane = vt_lane();
+#pragma unroll
+    for (int c = 0; c < NK; c++) {
+        const f32x4 *p = reinterpret_cast<const f32x4 *>(x + kofs + c * 512 + lane * 8);
+        xa[c] = p[0];
+        xb[c] = p[1];
+    }
+}
+
+/* RMSNorm of the full 3072-vector, every wave for itself (NK = 6 covers it):
+ * out = (x * 1/sqrt(mean(x^2)+eps)) * w  (voxtral_tts_kernels.c:333-349). */
+__device__ __forceinline__ void vt_rmsnorm_slice(f32x4 (&xa)[6], f32x4 (&xb)[6],
+                                                 const float *x, const float *w) {
+    vt_load_slice<6>(xa, xb, x, 0);
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < 6; c++) {
+        ss = fmaf(xa[c].x, xa[c].x, ss); ss = fmaf(xa[c].y, xa[c].y, ss);
+        ss = fmaf(xa[c].z, xa[c].z, ss); ss = fmaf(xa[c].w, xa[c].w, ss);
+        ss = fmaf(xb[c].x, xb[c].x, ss); ss = fmaf(xb[c].y, xb[c].y, ss);
+        ss = fmaf(xb[c].z, xb[c].z, ss); ss = fmaf(xb[c].w, xb[c].w, ss);
+    }
+    ss = vt_wave_sum(ss);
+    const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ss, (float)VT_DIM), VT_EPS)));
+    f32x4 wa[6], wb[6];
+    vt_load_slice<6>(wa, wb, w, 0);
+#pragma unroll
+    for (int c = 0; c < 6; c++) {
+        xa[c].x = __fmul_rn(__fmul_rn(xa[c].x, inv), wa[c].x);
+        xa[c].y = __fmul_rn(__fmul_rn(xa[c].y, inv), wa[c].y);
+        xa[c].z = __fmul_rn(__fmul_rn(xa[c].z, inv), wa[c].z);
+        xa[c].w = __fmul_rn(__fmul_rn(xa[c].w, inv), wa[c].w);
+        xb[c].x = __fmul_rn(__fmul_rn(xb[c].x, inv), wb[c].x);
+        xb[c].y = __fmul_rn(__fmul_rn(xb[c].y, inv), wb[c].y);
+        xb[c].z = __fmul_rn(__fmul_rn(xb[c].z, inv), wb[c].z);
+        xb[c].w = __fmul_rn(__fmul_rn(xb[c].w, inv), wb[c].w);
+    }
+}
+
+/* ---- row ring ------------------------------------------------------------- */
+
+/* Which rows of a phase a wave owns. */
+struct vt_rows {
+    int r0;        /* first global row of this wave (k-range [kofs, kofs+NK*512)) */
+    int nr;        /* rows owned by this wave (may be 0) */
+    int kofs;
+    int wg_row0;   /* first global row of the workgroup */
+    int wg_nrows;
+    int part;      /* k-split index of this wave */
+};
+
+/* Split `n_rows` rows over the grid (contiguous blocks, `align` rows granularity)
+ * and over the waves of the workgroup; KS waves share a row and split K. */
+template <int KS>
+__device__ __forceinline__ vt_rows vt_split_rows(int n_rows, int align, int k_per_part) {
+    vt_rows r;
+    const int G = (int)gridDim.x, wg = (int)blockIdx.x;
+    const int nw = (int)(blockDim.x >> 6), wave = vt_wave();
+    int per_wg = (n_rows + G - 1) / G;
+    per_wg = (per_wg + align - 1) / align * align;
+    r.wg_row0 = wg * per_wg;
+    int nrows = n_rows - r.wg_row0;
+    nrows = nrows < 0 ? 0 : (nrows > per_wg ? per_wg : nrows);
+    r.wg_nrows = nrows;
+    const int groups = nw / KS;
+    const int grp = wave / KS;
+    r.part = wave % KS;
+    const int per_grp = (nrows + groups - 1) / groups;
+    int g0 = grp * per_grp;
+    int gn = nrows - g0;
+    gn = gn < 0 ? 0 : (gn > per_grp ? per_grp : gn);
+    r.r0 = r.wg_row0 + g0;
+    r.nr = gn;
+    r.kofs = r.part * k_per_part;
+    return r;
+}
+
+/* Request the first D rows of a wave's share. */
+template <int NK, int D>
+__device__ __forceinline__ void vt_ring_prefetch(u32x4 (&ring)[VT_RING], const uint16_t *W,
+                                                 int row_len, const vt_rows &r) {
+    static_assert(NK * D <= VT_RING, "ring too small");
+    const uint16_t *base = W + (size_t)r.r0 * row_len + r.kofs + vt_lane() * 8;
+#pragma unroll
+    for (int j = 0; j < D; j++) {
+        if (j < r.nr) {
+#pragma unroll
+            for (int c = 0; c < NK; c++)
+                ring[j * NK + c] = vt_ldw(base + (size_t)j * row_len + c * 512);
+        }
+    }
+}
+
+/* Consume the wave's rows: y_lds[part * wg_nrows + local_row] = partial dot. */
+template <int NK, int D>
+__device__ __forceinline__ void vt_ring_run(u32x4 (&ring)[VT_RING], const uint16_t *W,
+                                            int row_len, const vt_rows &r,
+                                            const f32x4 (&xa)[NK], const f32x4 (&xb)[NK],
+                                            float *y_lds) {
+    const uint16_t *base = W + (size_t)r.r0 * row_len + r.kofs + vt_lane() * 8;
+    float *y = y_lds + r.part * r.wg_nrows + (r.r0 - r.wg_row0);
+    for (int i = 0; i < r.nr; i += D) {
+#pragma unroll
+        for (int j = 0; j < D; j++) {
+            const int row = i + j;
+            if (row < r.nr) {
+                float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+                for (int c = 0; c < NK; c += 2) {
+                    a0 = vt_dot8(ring[j * NK + c], xa[c], xb[c], a0);
+                    if (c + 1 < NK) a1 = vt_dot8(ring[j * NK + c + 1], xa[c + 1], xb[c + 1], a1);
+                }
+                if (row + D < r.nr) {
+#pragma unroll
+                    for (int c = 0; c < NK; c++)
+                        ring[j * NK + c] = vt_ldw(base + (size_t)(row + D) * row_len + c * 512);
+                }
+                const float s = vt_wave_sum(a0 + a1);
+                if (vt_lane() == 0) y[row] = s;
+            }
+        }
+    }
+}
+
+/* ---- phase 1: RMSNorm + [wq;wk;wv] + RoPE + cache append ------------------ */
+
+__device__ __forceinline__ vt_rows vt_qkv_rows() { return vt_split_rows<1>(VT_QKV_DIM, 2, 0); }
+
+__device__ __forceinline__ void vt_qkv_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L) {
+    vt_ring_prefetch<6, 3>(ring, L.wqkv, VT_DIM, vt_qkv_rows());
+}
+
+__device__ __forceinline__ void vt_qkv_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
+                                            const vt_step_args &a, int layer,
+                                            const float *x_in, float *lds) {
+    const vt_rows r = vt_qkv_rows();
+    f32x4 xa[6], xb[6];
+    vt_rmsnorm_slice(xa, xb, x_in, L.attn_norm);
+    vt_ring_run<6, 3>(ring, L.wqkv, VT_DIM, r, xa, xb, lds);
+    __syncthreads();
+    /* RoPE on adjacent pairs (voxtral_tts_kernels.c:616-634), then q to its
+     * buffer and k, v straight into row `pos` of the cache. */
+    const float *cs = a.rope + (size_t)a.pos * VT_HEAD_DIM;
+    const size_t kv_row = ((size_t)(a.first_layer + layer) * a.kv_max + a.pos) * VT_KV_DIM;
+    for (int t = (int)threadIdx.x; t < r.wg_nrows / 2; t += (int)blockDim.x) {
+        const int g = r.wg_row0 + 2 * t;
+        const float v0 = lds[2 * t], v1 = lds[2 * t + 1];
+        if (g < VT_Q_DIM + VT_KV_DIM) {
+            const int d = (g & (VT_HEAD_DIM - 1)) >> 1;
+            const float c = cs[2 * d], s = cs[2 * d + 1];
+            const float o0 = __fsub_rn(__fmul_rn(v0, c), __fmul_rn(v1, s));
+            const float o1 = __fadd_rn(__fmul_rn(v0, s), __fmul_rn(v1, c));
+            float *dst = g < VT_Q_DIM ? a.q + g : a.kv_k + kv_row + (g - VT_Q_DIM);
+            dst[0] = o0;
+            dst[1] = o1;
+        } else {
+            float *dst = a.kv_v + kv_row + (g - VT_Q_DIM - VT_KV_DIM);
+            dst[0] = v0;
+            dst[1] = v1;
+        }
+    }
+}
+
+/* ---- phase 2: GQA attention of one query over the cache ------------------- */
+/* Workgroup = (kv head, chunk of positions).  A wave walks its positions;
+ * lanes 16g..16g+15 serve query head 4*kvh+g and own 8 of the 128 dims.
+ * Partials (max, sum, o[128]) are merged over the waves in LDS, written per
+ * chunk, and the last workgroup to finish a kv head merges its chunks and
+ * normalises (online-softmax algebra of voxtral_tts_kernels.c:426-462). */
+__device__ __forceinline__ void vt_attn_phase(const vt_step_args &a, int layer, float *lds) {
+    const int G = (int)gridDim.x;
+    const int nch_max = G / VT_KV_HEADS;
+    const int wg = (int)blockIdx.x;
+    if (wg >= nch_max * VT_KV_HEADS) return;
+    const int kvh = wg % VT_KV_HEADS, chunk = wg / VT_KV_HEADS;
+    const int nw = (int)(blockDim.x >> 6), wave = vt_wave(), lane = vt_lane();
+    const int n = a.pos + 1;
+    int cs = (n + nch_max - 1) / nch_max;
+    cs = (cs + nw - 1) / nw * nw;
+    const int nch = (n + cs - 1) / cs;
+    if (chunk >= nch) return;
+    const int j0 = chunk * cs, j1 = min(n, j0 + cs);
+
+    const int grp = lane >> 4, sub = lane & 15;
+    const int head = kvh * 4 + grp;
+    const float scale = __fdiv_rn(1.0f, __fsqrt_rn((float)VT_HEAD_DIM));
+    const f32x4 *qp = reinterpret_cast<const f32x4 *>(a.q + head * VT_HEAD_DIM + sub * 8);
+    const f32x4 qa = qp[0], qb = qp[1];
+    const size_t layer_base = (size_t)(a.first_layer + layer) * a.kv_max * VT_KV_DIM;
+    const float *kbase = a.kv_k + layer_base + kvh * VT_HEAD_DIM + sub * 8;
+    const float *vbase = a.kv_v + layer_base + kvh * VT_HEAD_DIM + sub * 8;
+
+    float m = -1e30f, l = 0.f;
+    f32x4 oa = {0.f, 0.f, 0.f, 0.f}, ob = {0.f, 0.f, 0.f, 0.f};
+    for (int j = j0 + wave; j < j1; j += nw) {
+        const f32x4 *kp = reinterpret_cast<const f32x4 *>(kbase + (size_t)j * VT_KV_DIM);
+        const f32x4 *vp = reinterpret_cast<const f32x4 *>(vbase + (size_t)j * VT_KV_DIM);
+        const f32x4 ka = kp[0], kb = kp[1];
+        const f32x4 va = vp[0], vb = vp[1];
+        float s = qa.x * ka.x;
+        s = fmaf(qa.y, ka.y, s); s = fmaf(qa.z, ka.z, s); s = fmaf(qa.w, ka.w, s);
+        s = fmaf(qb.x, kb.x, s); s = fmaf(qb.y, kb.y, s); s = fmaf(qb.z, kb.z, s);
+        s = fmaf(qb.w, kb.w, s);
+        s = __fmul_rn(vt_row16_sum(s), scale);
+        const float mn = fmaxf(m, s);
+        const float corr = expf(m - mn), p = expf(s - mn);
+        l = fmaf(l, corr, p);
+        oa = oa * corr + va * p;
+        ob = ob * corr + vb * p;
+        m = mn;
+    }
+    /* merge the waves of this workgroup */
+    float *part = lds;                                   /* [nw][4][VT_ATT_STRIDE] */
+    float *mine = part + (wave * 4 + grp) * VT_ATT_STRIDE;
+    if (sub == 0) { mine[0] = m; mine[1] = l; }
+    *reinterpret_cast<f32x4 *>(mine + 4 + sub * 8) = oa;
+    *reinterpret_cast<f32x4 *>(mine + 8 + sub * 8) = ob;
+    __syncthreads();
+    for (int t = (int)threadIdx.x; t < 4 * VT_HEAD_DIM; t += (int)blockDim.x) {
+        const int g = t >> 7, d = t & 127;
+        float M = -1e30f;
+        for (int w = 0; w < nw; w++) M = fmaxf(M, part[(w * 4 + g) * VT_ATT_STRIDE]);
+        float Ls = 0.f, O = 0.f;
+        for (int w = 0; w < nw; w++) {
+            const float *pw = part + (w * 4 + g) * VT_ATT_STRIDE;
+            const float e = expf(pw[0] - M);
+            Ls = fmaf(pw[1], e, Ls);
+            O = fmaf(pw[4 + d], e, O);
+        }
+        float *dst = a.att_part + ((size_t)(kvh * 4 + g) * nch_max + chunk) * VT_ATT_STRIDE;
+        if (d == 0) { dst[0] = M; dst[1] = Ls; }
+        dst[4 + d] = O;
+    }
+    /* last workgroup of this kv head merges the chunks */
+    __shared__ int s_last;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned old = __hip_atomic_fetch_add(a.att_cnt + layer * VT_KV_HEADS + kvh, 1u,
+                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (old == (unsigned)(nch - 1));
+        if (s_last) __threadfence();
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (int t = (int)threadIdx.x; t < 4 * VT_HEAD_DIM; t += (int)blockDim.x) {
+        const int g = t >> 7, d = t & 127;
+        const float *src = a.att_part + (size_t)(kvh * 4 + g) * nch_max * VT_ATT_STRIDE;
+        float M = -1e30f;
+        for (int c = 0; c < nch; c++) M = fmaxf(M, vt_ld_coherent(src + c * VT_ATT_STRIDE));
+        float Ls = 0.f, O = 0.f;
+        for (int c = 0; c < nch; c++) {
+            const float e = expf(vt_ld_coherent(src + c * VT_ATT_STRIDE) - M);
+            Ls = fmaf(vt_ld_coherent(src + c * VT_ATT_STRIDE + 1), e, Ls);
+            O = fmaf(vt_ld_coherent(src + c * VT_ATT_STRIDE + 4 + d), e, O);
+        }
+        a.attn[(kvh * 4 + g) * VT_HEAD_DIM + d] = __fmul_rn(O, __fdiv_rn(1.0f, Ls));
+    }
+}
+
+/* ---- phase 3: x = x_in + wo * attn ---------------------------------------- */
+
+__device__ __forceinline__ vt_rows vt_wo_rows() { return vt_split_rows<2>(VT_DIM, 1, VT_Q_DIM / 2); }
+
+__device__ __forceinline__ void vt_wo_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L) {
+    vt_ring_prefetch<4, 4>(ring, L.wo, VT_Q_DIM, vt_wo_rows());
+}
+
+__device__ __forceinline__ void vt_wo_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
+                                           const vt_step_args &a, const float *x_in, float *lds) {
+    const vt_rows r = vt_wo_rows();
+    f32x4 xa[4], xb[4];
+    vt_load_slice<4>(xa, xb, a.attn, r.kofs);
+    vt_ring_run<4, 4>(ring, L.wo, VT_Q_DIM, r, xa, xb, lds);
+    __syncthreads();
+    for (int t = (int)threadIdx.x; t < r.wg_nrows; t += (int)blockDim.x) {
+        const float y = __fadd_rn(lds[t], lds[r.wg_nrows + t]);
+        a.x[r.wg_row0 + t] = __fadd_rn(x_in[r.wg_row0 + t], y);
+    }
+}
+
+/* ---- phase 4: RMSNorm + [w1|w3] + SiLU(gate)*up --------------------------- */
+
+__device__ __forceinline__ vt_rows vt_w13_rows() { return vt_split_rows<1>(2 * VT_FFN, 2, 0); }
+
+__device__ __forceinline__ void vt_w13_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L) {
+    vt_ring_prefetch<6, 3>(ring, L.w13, VT_DIM, vt_w13_rows());
+}
+
+__device__ __forceinline__ void vt_w13_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
+                                            const vt_step_args &a, float *lds) {
+    const vt_rows r = vt_w13_rows();
+    f32x4 xa[6], xb[6];
+    vt_rmsnorm_slice(xa, xb, a.x, L.ffn_norm);
+    vt_ring_run<6, 3>(ring, L.w13, VT_DIM, r, xa, xb, lds);
+    __syncthreads();
+    for (int t = (int)threadIdx.x; t < r.wg_nrows / 2; t += (int)blockDim.x) {
+        const float g = lds[2 * t], u = lds[2 * t + 1];
+        const float sg = __fdiv_rn(g, __fadd_rn(1.0f, expf(-g)));     /* voxtral_tts_kernels.c:361-366 */
+        a.h[r.wg_row0 / 2 + t] = __fmul_rn(sg, u);
+    }
+}
+
+/* ---- phase 5: x += w2 * h -------------------------------------------------- */
+
+__device__ __forceinline__ vt_rows vt_w2_rows() { return vt_split_rows<2>(VT_DIM, 1, VT_FFN / 2); }
+
+__device__ __forceinline__ void vt_w2_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L) {
+    vt_ring_prefetch<9, 2>(ring, L.w2, VT_FFN, vt_w2_rows());
+}
+
+__device__ __forceinline__ void vt_w2_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
+                                           const vt_step_args &a, float *lds) {
+    const vt_rows r = vt_w2_rows();
+    f32x4 xa[9], xb[9];
+    vt_load_slice<9>(xa, xb, a.h, r.kofs);
+    vt_ring_run<9, 2>(ring, L.w2, VT_FFN, r, xa, xb, lds);
+    __syncthreads();
+    for (int t = (int)threadIdx.x; t < r.wg_nrows; t += (int)blockDim.x) {
+        const float y = __fadd_rn(lds[t], lds[r.wg_nrows + t]);
+        a.x[r.wg_row0 + t] = __fadd_rn(a.x[r.wg_row0 + t], y);
+    }
+}
+
+/* ---- final RMSNorm (one workgroup) ----------------------------------------- */
+
+__device__ __forceinline__ void vt_block_rmsnorm(float *out, const float *x, const float *w,
+                                                 int dim, float eps, float *lds) {
+    float ss = 0.f;
+    for (int i = (int)threadIdx.x; i < dim; i += (int)blockDim.x) ss = fmaf(x[i], x[i], ss);
+    ss = vt_wave_sum(ss);
+    if (vt_lane() == 0) lds[vt_wave()] = ss;
+    __syncthreads();
+    float tot = 0.f;
+    for (int w_ = 0; w_ < (int)(blockDim.x >> 6); w_++) tot += lds[w_];
+    const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(tot, (float)dim), eps)));
+    for (int i = (int)threadIdx.x; i < dim; i += (int)blockDim.x)
+        out[i] = __fmul_rn(__fmul_rn(x[i], inv), w[i]);
+    __syncthreads();
+}
+
+#endif /* VT_DECODE_PHASES_H */

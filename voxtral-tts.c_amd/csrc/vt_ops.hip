@@ -1,0 +1,317 @@
+/*
+ * vt_ops.hip - kernel-level operators of the C ABI on device pointers
+ * (replace the standalone kernels of voxtral_tts_cuda.cu:331-704): generic
+ * bf16-weight linear, RMSNorm, RoPE, SiLU*mul, residual add, attention
+ * (decode / causal prefill / bidirectional) and embedding lookup.
+ * Shapes are arbitrary here; the fixed-shape fused paths live in
+ * vt_decode.hip / vt_prefill.hip / vt_acoustic.hip.
+ */
+#include "vt_state.h"
+
+#include <math.h>
+#include <stdlib.h>
+
+/* ---- linear: y[s,o] = bias[o] + sum_k W[o,k] x[s,k] ------------------------- */
+/* One wave per output row; up to S rows of x share each weight load. */
+template <int S>
+__global__ void __launch_bounds__(256)
+vt_linear_kernel(float *y, const float *x, const uint16_t *W, const float *bias,
+                 int seq_len, int in_dim, int out_dim, int vec_ok) {
+    const int row = (int)blockIdx.x * (int)(blockDim.x >> 6) + vt_wave();
+    if (row >= out_dim) return;
+    const int lane = vt_lane();
+    const uint16_t *wr = W + (size_t)row * in_dim;
+    for (int s0 = 0; s0 < seq_len; s0 += S) {
+        float acc[S];
+#pragma unroll
+        for (int s = 0; s < S; s++) acc[s] = 0.f;
+        if (vec_ok) {
+            for (int k = lane * 8; k < in_dim; k += 512) {
+                const u32x4 w = *reinterpret_cast<const u32x4 *>(wr + k);
+#pragma unroll
+                for (int s = 0; s < S; s++) {
+                    if (s0 + s < seq_len) {
+                        const f32x4 *xp = reinterpret_cast<const f32x4 *>(x + (size_t)(s0 + s) * in_dim + k);
+                        acc[s] = vt_dot8(w, xp[0], xp[1], acc[s]);
+                    }
+                }
+            }
+        } else {
+            for (int k = lane; k < in_dim; k += 64) {
+                const float w = __uint_as_float((unsigned)wr[k] << 16);
+#pragma unroll
+                for (int s = 0; s < S; s++)
+                    if (s0 + s < seq_len) acc[s] = fmaf(w, x[(size_t)(s0 + s) * in_dim + k], acc[s]);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            const float v = vt_wave_sum(acc[s]);
+            if (lane == 0 && s0 + s < seq_len)
+                y[(size_t)(s0 + s) * out_dim + row] = bias ? __fadd_rn(bias[row], v) : v;
+        }
+    }
+}
+
+void vt_launch_linear(float *d_y, const float *d_x, const uint16_t *d_W, const float *d_bias,
+                      int seq_len, int in_dim, int out_dim) {
+    const int vec_ok = (in_dim % 8 == 0) && (((uintptr_t)d_W | (uintptr_t)d_x) % 16 == 0);
+    const dim3 grid((out_dim + 3) / 4), block(256);
+    if (seq_len == 1)
+        hipLaunchKernelGGL(vt_linear_kernel<1>, grid, block, 0, g_vt.stream, d_y, d_x, d_W, d_bias,
+                           seq_len, in_dim, out_dim, vec_ok);
+    else if (seq_len <= 4)
+        hipLaunchKernelGGL(vt_linear_kernel<4>, grid, block, 0, g_vt.stream, d_y, d_x, d_W, d_bias,
+                           seq_len, in_dim, out_dim, vec_ok);
+    else
+        hipLaunchKernelGGL(vt_linear_kernel<8>, grid, block, 0, g_vt.stream, d_y, d_x, d_W, d_bias,
+                           seq_len, in_dim, out_dim, vec_ok);
+}
+
+static int is_device_ptr(const void *p) {
+    hipPointerAttribute_t at;
+    if (hipPointerGetAttributes(&at, p) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return at.type == hipMemoryTypeDevice;
+}
+
+extern "C" void tts_hip_linear_bf16(float *y, const float *x, const uint16_t *W_bf16,
+                                    int seq_len, int in_dim, int out_dim, const void *W_gpu) {
+    if (!g_vt.initialized) { vt_set_error("tts_hip_linear_bf16: backend not initialised"); return; }
+    if (seq_len < 1 || in_dim < 1 || out_dim < 1) { vt_set_error("tts_hip_linear_bf16: bad shape"); return; }
+    const size_t xb = sizeof(float) * (size_t)seq_len * in_dim, yb = sizeof(float) * (size_t)seq_len * out_dim;
+    const size_t wb = 2 * (size_t)out_dim * in_dim;
+    const int x_dev = is_device_ptr(x), y_dev = is_device_ptr(y);
+    float *dx = (float *)x, *dy = y;
+    void *dW = (void *)W_gpu, *tmp_x = NULL, *tmp_y = NULL, *tmp_W = NULL;
+    if (!x_dev) {
+        if (!(tmp_x = vt_dev_alloc(xb))) return;
+        if (vt_check(hipMemcpy(tmp_x, x, xb, hipMemcpyHostToDevice), "linear x upload")) goto done;
+        dx = (float *)tmp_x;
+    }
+    if (!dW) {
+        if (!W_bf16) { vt_set_error("tts_hip_linear_bf16: no weights given"); goto done; }
+        if (!(tmp_W = vt_dev_alloc(wb))) goto done;
+        if (vt_check(hipMemcpy(tmp_W, W_bf16, wb, hipMemcpyHostToDevice), "linear W upload")) goto done;
+        dW = tmp_W;
+    }
+    if (!y_dev) {
+        if (!(tmp_y = vt_dev_alloc(yb))) goto done;
+        dy = (float *)tmp_y;
+    }
+    vt_launch_linear(dy, dx, (const uint16_t *)dW, NULL, seq_len, in_dim, out_dim);
+    if (!y_dev || tmp_x || tmp_W) {
+        if (vt_check(hipStreamSynchronize(g_vt.stream), "linear sync")) goto done;
+        if (!y_dev) (void)vt_check(hipMemcpy(y, dy, yb, hipMemcpyDeviceToHost), "linear y download");
+    }
+done:
+    if (tmp_x) (void)hipFree(tmp_x);
+    if (tmp_y) (void)hipFree(tmp_y);
+    if (tmp_W) (void)hipFree(tmp_W);
+}
+
+/* ---- RMSNorm: one workgroup per row ------------------------------------------ */
+
+__global__ void __launch_bounds__(256)
+vt_rms_norm_kernel(float *out, const float *x, const float *w, int dim, float eps) {
+    __shared__ float lds[VT_MAX_WAVES];
+    vt_block_rmsnorm(out + (size_t)blockIdx.x * dim, x + (size_t)blockIdx.x * dim, w, dim, eps, lds);
+}
+
+void vt_launch_rms_norm(float *d_out, const float *d_x, const float *d_w, int seq, int dim, float eps) {
+    hipLaunchKernelGGL(vt_rms_norm_kernel, dim3(seq), dim3(256), 0, g_vt.stream, d_out, d_x, d_w, dim, eps);
+}
+
+extern "C" void tts_hip_rms_norm(float *d_out, const float *d_x, const float *d_weight,
+                                 int seq_len, int dim, float eps) {
+    if (!g_vt.initialized || seq_len < 1 || dim < 1) { vt_set_error("tts_hip_rms_norm: bad call"); return; }
+    vt_launch_rms_norm(d_out, d_x, d_weight, seq_len, dim, eps);
+}
+
+/* ---- RoPE on adjacent pairs with a (cos, sin) table ---------------------------- */
+
+__global__ void vt_rope_kernel(float *x, const float *freqs, int seq, int heads, int head_dim) {
+    const int half = head_dim / 2;
+    const size_t total = (size_t)seq * heads * half;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        const int d = (int)(i % half);
+        const size_t sh = i / half;
+        const int s = (int)(sh / heads);
+        const float c = freqs[((size_t)s * half + d) * 2], sn = freqs[((size_t)s * half + d) * 2 + 1];
+        float *v = x + sh * head_dim + 2 * d;
+        const float a = v[0], b = v[1];
+        v[0] = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn));
+        v[1] = __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c));
+    }
+}
+
+extern "C" void tts_hip_apply_rope(float *d_x, const float *d_freqs, int seq, int heads, int head_dim) {
+    if (!g_vt.initialized || seq < 1 || heads < 1 || head_dim < 2 || (head_dim & 1)) {
+        vt_set_error("tts_hip_apply_rope: bad call");
+        return;
+    }
+    const size_t total = (size_t)seq * heads * (head_dim / 2);
+    const int blocks = (int)((total + 255) / 256 > 4096 ? 4096 : (total + 255) / 256);
+    hipLaunchKernelGGL(vt_rope_kernel, dim3(blocks), dim3(256), 0, g_vt.stream, d_x, d_freqs, seq, heads, head_dim);
+}
+
+/* The table is evaluated on the host with libm in the operation order of
+ * voxtral_tts_kernels.c:602-614, then copied: entries are bit-equal to the CPU path. */
+extern "C" void tts_hip_compute_rope_freqs(float *d_freqs, int start_pos, int seq, int dim, float theta) {
+    if (!g_vt.initialized || seq < 1 || dim < 2) { vt_set_error("tts_hip_compute_rope_freqs: bad call"); return; }
+    const int half = dim / 2;
+    float *t = (float *)malloc(sizeof(float) * (size_t)seq * half * 2);
+    if (!t) { vt_set_error("tts_hip_compute_rope_freqs: out of host memory"); return; }
+    for (int s = 0; s < seq; s++) {
+        const float p = (float)(start_pos + s);
+        for (int d = 0; d < half; d++) {
+            const float f = 1.0f / powf(theta, (float)(2 * d) / (float)dim);
+            volatile float ang = p * f;
+            t[((size_t)s * half + d) * 2] = cosf(ang);
+            t[((size_t)s * half + d) * 2 + 1] = sinf(ang);
+        }
+    }
+    (void)hipStreamSynchronize(g_vt.stream);
+    (void)vt_check(hipMemcpy(d_freqs, t, sizeof(float) * (size_t)seq * half * 2, hipMemcpyHostToDevice),
+                   "rope table copy");
+    free(t);
+}
+
+/* ---- SiLU(gate) * up, residual add --------------------------------------------- */
+
+__global__ void vt_silu_mul_kernel(float *gate, const float *up, int n) {
+    for (int i = (int)(blockIdx.x * blockDim.x + threadIdx.x); i < n; i += (int)(gridDim.x * blockDim.x)) {
+        const float g = gate[i];
+        gate[i] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), up[i]);
+    }
+}
+
+__global__ void vt_add_kernel(float *a, const float *b, int n) {
+    for (int i = (int)(blockIdx.x * blockDim.x + threadIdx.x); i < n; i += (int)(gridDim.x * blockDim.x))
+        a[i] = __fadd_rn(a[i], b[i]);
+}
+
+static int ew_blocks(int n) { int b = (n + 255) / 256; return b > 2048 ? 2048 : b; }
+
+extern "C" void tts_hip_silu_mul(float *d_gate, const float *d_up, int n) {
+    if (!g_vt.initialized || n < 1) { vt_set_error("tts_hip_silu_mul: bad call"); return; }
+    hipLaunchKernelGGL(vt_silu_mul_kernel, dim3(ew_blocks(n)), dim3(256), 0, g_vt.stream, d_gate, d_up, n);
+}
+
+void vt_launch_add(float *d_a, const float *d_b, int n) {
+    hipLaunchKernelGGL(vt_add_kernel, dim3(ew_blocks(n)), dim3(256), 0, g_vt.stream, d_a, d_b, n);
+}
+
+extern "C" void tts_hip_add_inplace(float *d_a, const float *d_b, int n) {
+    if (!g_vt.initialized || n < 1) { vt_set_error("tts_hip_add_inplace: bad call"); return; }
+    vt_launch_add(d_a, d_b, n);
+}
+
+/* ---- attention, any head geometry (head_dim <= 256, multiple of 64) ------------- */
+/* Workgroup = (head, query).  Waves stride over the keys, each lane owns
+ * head_dim/64 dims; per-wave online softmax, merged over the waves in LDS.
+ * Keys visible to query i: [0, min(q_offset+i+1, seq_k)) when causal, else all. */
+__global__ void __launch_bounds__(256)
+vt_attention_kernel(float *out, const float *Q, const float *K, const float *V, int q_offset,
+                    int seq_k, int causal, int n_heads, int n_kv_heads, int head_dim,
+                    float scale, int kv_stride, int q_stride) {
+    __shared__ float part[4][2 + 256];
+    const int h = (int)blockIdx.x, i = (int)blockIdx.y;
+    const int kvh = h / (n_heads / n_kv_heads);
+    const int lane = vt_lane(), wave = vt_wave(), nw = (int)(blockDim.x >> 6);
+    const int per = head_dim / 64;
+    int kend = seq_k;
+    if (causal) { kend = q_offset + i + 1; if (kend > seq_k) kend = seq_k; }
+    const float *q = Q + (size_t)i * q_stride + (size_t)h * head_dim;
+    float qv[4], o[4];
+    for (int e = 0; e < 4; e++) { qv[e] = e < per ? q[lane + 64 * e] : 0.f; o[e] = 0.f; }
+    float m = -1e30f, l = 0.f;
+    for (int j = wave; j < kend; j += nw) {
+        const float *kr = K + (size_t)j * kv_stride + kvh * head_dim;
+        const float *vr = V + (size_t)j * kv_stride + kvh * head_dim;
+        float s = 0.f;
+        for (int e = 0; e < per; e++) s = fmaf(qv[e], kr[lane + 64 * e], s);
+        s = __fmul_rn(vt_wave_sum(s), scale);
+        const float mn = fmaxf(m, s);
+        const float corr = expf(m - mn), p = expf(s - mn);
+        l = fmaf(l, corr, p);
+        for (int e = 0; e < per; e++) o[e] = fmaf(o[e], corr, p * vr[lane + 64 * e]);
+        m = mn;
+    }
+    if (lane == 0) { part[wave][0] = m; part[wave][1] = l; }
+    for (int e = 0; e < per; e++) part[wave][2 + lane + 64 * e] = o[e];
+    __syncthreads();
+    for (int d = (int)threadIdx.x; d < head_dim; d += (int)blockDim.x) {
+        float M = -1e30f;
+        for (int w = 0; w < nw; w++) M = fmaxf(M, part[w][0]);
+        float L = 0.f, O = 0.f;
+        for (int w = 0; w < nw; w++) {
+            const float e = expf(part[w][0] - M);
+            L = fmaf(part[w][1], e, L);
+            O = fmaf(part[w][2 + d], e, O);
+        }
+        out[((size_t)i * n_heads + h) * head_dim + d] = L > 0.f ? __fmul_rn(O, __fdiv_rn(1.0f, L)) : 0.f;
+    }
+}
+
+void vt_launch_attention(float *d_out, const float *d_Q, const float *d_K, const float *d_V,
+                         int seq_q, int q_offset, int seq_k, int causal, int n_heads,
+                         int n_kv_heads, int head_dim, float scale, int kv_stride, int q_stride) {
+    hipLaunchKernelGGL(vt_attention_kernel, dim3(n_heads, seq_q), dim3(256), 0, g_vt.stream, d_out, d_Q,
+                       d_K, d_V, q_offset, seq_k, causal, n_heads, n_kv_heads, head_dim, scale, kv_stride,
+                       q_stride);
+}
+
+static int attn_args_ok(const char *who, int seq_q, int seq_k, int n_heads, int n_kv_heads, int head_dim) {
+    if (g_vt.initialized && seq_q >= 1 && seq_k >= 1 && n_heads >= 1 && n_kv_heads >= 1 &&
+        n_heads % n_kv_heads == 0 && head_dim >= 64 && head_dim <= 256 && head_dim % 64 == 0)
+        return 1;
+    vt_set_error("%s: unsupported arguments (heads %d/%d, head_dim %d, seq %d/%d)", who, n_heads,
+                 n_kv_heads, head_dim, seq_q, seq_k);
+    return 0;
+}
+
+extern "C" void tts_hip_causal_attention_decode(float *d_out, const float *d_Q, const float *d_K_cache,
+                                                const float *d_V_cache, int seq_k, int n_heads,
+                                                int n_kv_heads, int head_dim, float scale,
+                                                int kv_cache_stride) {
+    if (!attn_args_ok("tts_hip_causal_attention_decode", 1, seq_k, n_heads, n_kv_heads, head_dim)) return;
+    const int stride = kv_cache_stride > 0 ? kv_cache_stride : n_kv_heads * head_dim;
+    vt_launch_attention(d_out, d_Q, d_K_cache, d_V_cache, 1, seq_k - 1, seq_k, 1, n_heads, n_kv_heads,
+                        head_dim, scale, stride, n_heads * head_dim);
+}
+
+extern "C" void tts_hip_causal_attention_prefill(float *d_out, const float *d_Q, const float *d_K,
+                                                 const float *d_V, int seq_len, int start_pos,
+                                                 int n_heads, int n_kv_heads, int head_dim, float scale) {
+    if (!attn_args_ok("tts_hip_causal_attention_prefill", seq_len, start_pos + seq_len, n_heads,
+                      n_kv_heads, head_dim)) return;
+    if (start_pos < 0) { vt_set_error("tts_hip_causal_attention_prefill: negative start_pos"); return; }
+    vt_launch_attention(d_out, d_Q, d_K, d_V, seq_len, start_pos, start_pos + seq_len, 1, n_heads,
+                        n_kv_heads, head_dim, scale, n_kv_heads * head_dim, n_heads * head_dim);
+}
+
+extern "C" void tts_hip_bidirectional_attention(float *d_out, const float *d_Q, const float *d_K,
+                                                const float *d_V, int seq_len, int n_heads,
+                                                int n_kv_heads, int head_dim, float scale) {
+    if (!attn_args_ok("tts_hip_bidirectional_attention", seq_len, seq_len, n_heads, n_kv_heads, head_dim))
+        return;
+    vt_launch_attention(d_out, d_Q, d_K, d_V, seq_len, 0, seq_len, 0, n_heads, n_kv_heads, head_dim,
+                        scale, n_kv_heads * head_dim, n_heads * head_dim);
+}
+
+/* ---- embedding lookup ------------------------------------------------------------ */
+
+__global__ void vt_embed_kernel(float *out, const uint16_t *emb, int token_id, int dim) {
+    const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (i < dim) out[i] = __uint_as_float((unsigned)emb[(size_t)token_id * dim + i] << 16);
+}
+
+extern "C" void tts_hip_embed_token(float *d_out, const void *d_embeddings_bf16, int token_id, int dim) {
+    if (!g_vt.initialized || token_id < 0 || dim < 1) { vt_set_error("tts_hip_embed_token: bad call"); return; }
+    hipLaunchKernelGGL(vt_embed_kernel, dim3((dim + 255) / 256), dim3(256), 0, g_vt.stream, d_out,
+                       (const uint16_t *)d_embeddings_bf16, token_id, dim);
+}

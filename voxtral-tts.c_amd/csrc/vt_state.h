@@ -1,0 +1,95 @@
+/*
+ * vt_state.h - host-side state of the backend (one global context, as in the
+ * reference backend: voxtral_tts_cuda.cu:56) and the helpers shared by the
+ * translation units of the library.
+ */
+#ifndef VT_STATE_H
+#define VT_STATE_H
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "../../include/voxtral_tts_hip.h"
+#include "vt_decode_phases.h"
+
+#define VT_MAX_WAVES 8
+#define VT_STEP_THREADS 512
+#define VT_ATT_LDS_FLOATS (VT_MAX_WAVES * 4 * VT_ATT_STRIDE)
+#define VT_AC_SEQ 3
+#define VT_AC_DIM_IN 36
+#define VT_SEM_PADDED 8320
+#define VT_SEM_VALID_END 8194     /* 2 special + 8192 codes */
+
+struct vt_acoustic_dev {
+    vt_layer_dev layers[TTS_HIP_AC_LAYERS];
+    uint16_t *input_proj, *time_proj, *llm_proj, *semantic_out, *acoustic_out;
+    float *semantic_bias;         /* NULL when the checkpoint has none */
+    float *norm;
+    float *time_inv_freq;
+    float h_time_inv_freq[VT_DIM / 2];
+};
+
+struct vt_state {
+    int initialized;
+    int device;
+    int n_cu;
+    int grid;                     /* workgroups of the persistent kernels */
+    size_t step_dyn_lds;          /* dynamic LDS that pins one workgroup per CU */
+    hipStream_t stream;
+    hipEvent_t ev0, ev1;
+    int decode_mode;
+
+    /* backbone weights */
+    vt_layer_dev h_layers[TTS_HIP_DEC_LAYERS];
+    vt_layer_dev *d_layers;
+    float *d_dec_norm;
+    uint16_t *d_tok_emb;
+    int n_dec_layers;
+
+    /* acoustic weights */
+    vt_acoustic_dev ac;
+    int ac_uploaded;
+
+    /* caches and tables */
+    float *d_rope;                /* [kv_max, 64, 2] */
+    int kv_max;
+
+    /* decode work buffers */
+    float *d_x, *d_q, *d_attn, *d_h, *d_att_part, *d_embed, *d_hidden;
+    unsigned int *d_att_cnt;
+    unsigned long long *d_bar_counter;
+    unsigned long long bar_base;
+    int *d_abort;
+    float *h_pin;                 /* pinned staging: [3072 in][3072 out + flag] */
+
+    /* generic scratch (prefill / acoustic / linear) */
+    void *d_scratch;
+    size_t scratch_bytes;
+
+    int error_count;
+    char last_error[512];
+};
+
+extern vt_state g_vt;
+
+void vt_set_error(const char *fmt, ...);
+int vt_check(hipError_t e, const char *what);
+void *vt_scratch(size_t bytes);      /* grows on demand; contents undefined */
+void *vt_dev_alloc(size_t bytes);
+
+#define VT_TRY(call) do { if (vt_check((call), #call)) return -1; } while (0)
+#define VT_TRYV(call) do { if (vt_check((call), #call)) return; } while (0)
+
+/* kernels launched from other translation units */
+void vt_launch_linear(float *d_y, const float *d_x, const uint16_t *d_W, const float *d_bias,
+                      int seq_len, int in_dim, int out_dim);
+void vt_launch_rms_norm(float *d_out, const float *d_x, const float *d_w, int seq, int dim, float eps);
+void vt_launch_attention(float *d_out, const float *d_Q, const float *d_K, const float *d_V,
+                         int seq_q, int q_offset, int seq_k, int causal, int n_heads,
+                         int n_kv_heads, int head_dim, float scale, int kv_stride, int q_stride);
+void vt_launch_add(float *d_a, const float *d_b, int n);
+int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
+                const float *d_final_norm, const float *d_in, float *d_out, int pos);
+
+#endif /* VT_STATE_H */
