@@ -126,14 +126,14 @@ extern "C" int tts_hip_init(int kv_cache_max) {
         {(void **)&g_vt.d_att_cnt, sizeof(unsigned) * TTS_HIP_DEC_LAYERS * VT_KV_HEADS},
         {(void **)&g_vt.d_embed, sizeof(float) * VT_DIM},
         {(void **)&g_vt.d_hidden, sizeof(float) * (VT_DIM + 64)},
-        {(void **)&g_vt.d_bar_counter, 256},
+        {(void **)&g_vt.d_bar_flags, sizeof(unsigned) * (size_t)g_vt.grid + 256},
         {(void **)&g_vt.d_abort, 256},
     };
     for (size_t i = 0; i < sizeof bufs / sizeof bufs[0]; i++) {
         if (!(*bufs[i].p = vt_dev_alloc(bufs[i].bytes))) return -1;
         VT_TRY(hipMemset(*bufs[i].p, 0, bufs[i].bytes));
     }
-    g_vt.bar_base = 0;
+    g_vt.bar_epoch = 0;
     VT_TRY(hipHostMalloc((void **)&g_vt.h_pin, sizeof(float) * (2 * VT_DIM + 64), hipHostMallocDefault));
     VT_TRY(hipDeviceSynchronize());
 
@@ -159,7 +159,7 @@ extern "C" void tts_hip_free(void) {
                     g_vt.ac.acoustic_out, g_vt.ac.semantic_bias, g_vt.ac.norm,
                     g_vt.ac.time_inv_freq, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu,
                     g_vt.d_rope, g_vt.d_x, g_vt.d_q, g_vt.d_attn, g_vt.d_h, g_vt.d_att_part,
-                    g_vt.d_att_cnt, g_vt.d_embed, g_vt.d_hidden, g_vt.d_bar_counter,
+                    g_vt.d_att_cnt, g_vt.d_embed, g_vt.d_hidden, g_vt.d_bar_flags,
                     g_vt.d_abort, g_vt.d_scratch};
     for (size_t i = 0; i < sizeof ptrs / sizeof ptrs[0]; i++)
         if (ptrs[i]) (void)hipFree(ptrs[i]);

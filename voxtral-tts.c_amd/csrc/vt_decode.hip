@@ -17,43 +17,24 @@
 
 /* ---- persistent whole-step kernel -------------------------------------------- */
 
+/* Arrive at the grid barrier, request the next phase's first weight rows while
+ * the other workgroups arrive, then wait. */
 template <class F>
 __device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between) {
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        __threadfence();
-        __hip_atomic_fetch_add(gs.counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    between();                      /* request the next phase's first weight rows */
-    if (threadIdx.x == 0) {
-        int ok = 1;
-        const unsigned long long t0 = wall_clock64();
-        while (__hip_atomic_load(gs.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gs.target) {
-            __builtin_amdgcn_s_sleep(1);
-            if (__hip_atomic_load(gs.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
-                wall_clock64() - t0 > gs.timeout) {
-                __hip_atomic_store(gs.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                ok = 0;
-                break;
-            }
-        }
-        __threadfence();
-        *flag = ok;
-    }
-    __syncthreads();
-    gs.target += gridDim.x;
-    return *flag != 0;
+    vt_barrier_arrive(gs);
+    between();
+    return vt_barrier_wait(gs, flag);
 }
 
 __global__ void __launch_bounds__(VT_STEP_THREADS)
 vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
-    __shared__ __attribute__((aligned(16))) float lds[VT_ATT_LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds[VT_LDS_FLOATS];
     __shared__ int s_flag;
     u32x4 ring[VT_RING];
 
     if (blockIdx.x == 0)
         for (int t = (int)threadIdx.x; t < a.n_layers * VT_KV_HEADS; t += (int)blockDim.x)
-            a.att_cnt[t] = 0u;
+            vt_stc_u32(a.att_cnt + t, 0u);
 
     const float *x_in = a.in_embed;
     vt_qkv_prefetch(ring, a.layers[0]);
@@ -75,9 +56,9 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
     }
     if (blockIdx.x == 0) {
         if (a.final_norm) {
-            vt_block_rmsnorm(a.out_hidden, a.x, a.final_norm, VT_DIM, VT_EPS, lds);
+            vt_block_rmsnorm<true>(a.out_hidden, a.x, a.final_norm, VT_DIM, VT_EPS, lds);
         } else {
-            for (int i = (int)threadIdx.x; i < VT_DIM; i += (int)blockDim.x) a.out_hidden[i] = a.x[i];
+            for (int i = (int)threadIdx.x; i < VT_DIM; i += (int)blockDim.x) a.out_hidden[i] = vt_ldc(a.x + i);
         }
     }
 }
@@ -86,7 +67,7 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
 
 __global__ void __launch_bounds__(VT_STEP_THREADS)
 vt_qkv_kernel(vt_step_args a, int l, const float *x_in) {
-    __shared__ __attribute__((aligned(16))) float lds[256];
+    __shared__ __attribute__((aligned(16))) float lds[VT_LDS_FLOATS];
     u32x4 ring[VT_RING];
     const vt_layer_dev L = a.layers[l];
     vt_qkv_prefetch(ring, L);
@@ -95,13 +76,13 @@ vt_qkv_kernel(vt_step_args a, int l, const float *x_in) {
 
 __global__ void __launch_bounds__(VT_STEP_THREADS)
 vt_attn_kernel(vt_step_args a, int l) {
-    __shared__ __attribute__((aligned(16))) float lds[VT_ATT_LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float lds[VT_LDS_FLOATS];
     vt_attn_phase(a, l, lds);
 }
 
 __global__ void __launch_bounds__(VT_STEP_THREADS)
 vt_wo_kernel(vt_step_args a, int l, const float *x_in) {
-    __shared__ __attribute__((aligned(16))) float lds[256];
+    __shared__ __attribute__((aligned(16))) float lds[VT_LDS_FLOATS];
     u32x4 ring[VT_RING];
     const vt_layer_dev L = a.layers[l];
     vt_wo_prefetch(ring, L);
@@ -110,7 +91,7 @@ vt_wo_kernel(vt_step_args a, int l, const float *x_in) {
 
 __global__ void __launch_bounds__(VT_STEP_THREADS)
 vt_w13_kernel(vt_step_args a, int l) {
-    __shared__ __attribute__((aligned(16))) float lds[256];
+    __shared__ __attribute__((aligned(16))) float lds[VT_LDS_FLOATS];
     u32x4 ring[VT_RING];
     const vt_layer_dev L = a.layers[l];
     vt_w13_prefetch(ring, L);
@@ -119,7 +100,7 @@ vt_w13_kernel(vt_step_args a, int l) {
 
 __global__ void __launch_bounds__(VT_STEP_THREADS)
 vt_w2_kernel(vt_step_args a, int l) {
-    __shared__ __attribute__((aligned(16))) float lds[256];
+    __shared__ __attribute__((aligned(16))) float lds[VT_LDS_FLOATS];
     u32x4 ring[VT_RING];
     const vt_layer_dev L = a.layers[l];
     vt_w2_prefetch(ring, L);
@@ -130,7 +111,7 @@ __global__ void __launch_bounds__(VT_STEP_THREADS)
 vt_final_kernel(vt_step_args a) {
     __shared__ float lds[VT_MAX_WAVES];
     if (a.final_norm) {
-        vt_block_rmsnorm(a.out_hidden, a.x, a.final_norm, VT_DIM, VT_EPS, lds);
+        vt_block_rmsnorm<false>(a.out_hidden, a.x, a.final_norm, VT_DIM, VT_EPS, lds);
     } else {
         for (int i = (int)threadIdx.x; i < VT_DIM; i += (int)blockDim.x) a.out_hidden[i] = a.x[i];
     }
@@ -181,11 +162,11 @@ int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
     hipStream_t st = g_vt.stream;
     if (g_vt.decode_mode == 0) {
         vt_grid_sync gs;
-        gs.counter = g_vt.d_bar_counter;
+        gs.flags = g_vt.d_bar_flags;
         gs.abort_flag = g_vt.d_abort;
-        gs.target = g_vt.bar_base + (unsigned long long)g_vt.grid;
+        gs.epoch = g_vt.bar_epoch + 1u;
         gs.timeout = 20000000ull;                 /* 0.2 s of the 100 MHz wall clock */
-        g_vt.bar_base += (unsigned long long)g_vt.grid * 5ull * (unsigned long long)n_layers;
+        g_vt.bar_epoch += 5u * (unsigned)n_layers;
         static int attr_set = 0;
         if (!attr_set && g_vt.step_dyn_lds) {
             if (vt_check(hipFuncSetAttribute((const void *)vt_decode_step_kernel,
@@ -217,9 +198,9 @@ static int step_aborted(int flag) {
     if (!flag) return 0;
     vt_set_error("decode step: grid barrier timed out; kernel left early, result invalid");
     (void)hipMemsetAsync(g_vt.d_abort, 0, sizeof(int), g_vt.stream);
-    (void)hipMemsetAsync(g_vt.d_bar_counter, 0, sizeof(unsigned long long), g_vt.stream);
+    (void)hipMemsetAsync(g_vt.d_bar_flags, 0, sizeof(unsigned) * g_vt.grid, g_vt.stream);
     (void)hipStreamSynchronize(g_vt.stream);
-    g_vt.bar_base = 0;
+    g_vt.bar_epoch = 0;
     return -1;
 }
 

@@ -12,6 +12,12 @@
  * per wave; the first D rows of a phase can be requested before the grid
  * barrier that precedes the phase (weights do not depend on activations).
  *
+ * The small vectors that one phase hands to the next (residual stream, q,
+ * attention output, SwiGLU output, the appended K/V row, attention partials)
+ * cross workgroups and therefore XCDs: they are written through to memory
+ * (vt_stc) and read past the L2 (vt_ldc / vt_stage), once per workgroup into
+ * LDS, from where every wave takes its register slice.
+ *
  * Operation order follows the reference CPU decode step
  * (voxtral_tts_llm.c:205-264): RMSNorm -> q,k,v -> RoPE -> cache append ->
  * attention -> wo + residual -> RMSNorm -> w1,w3 -> SiLU*up -> w2 + residual.
@@ -23,6 +29,10 @@
 
 #define VT_RING 18            /* 16-byte buffers per lane in the row ring */
 #define VT_ATT_STRIDE 132     /* floats per attention partial: m, l, pad, pad, o[128] */
+#define VT_ATT_MIN_CHUNK 128  /* positions per attention workgroup before the cache is split further */
+#define VT_LDS_X 9216         /* staged activation vector (largest: the SwiGLU output) */
+#define VT_LDS_Y 512          /* row results of one workgroup */
+#define VT_LDS_FLOATS (VT_LDS_X + VT_LDS_Y)
 
 /* Device-side weights of one layer, laid out at upload:
  *   wqkv = [wq ; wk ; wv]            [6144, 3072]
@@ -53,11 +63,38 @@ struct vt_step_args {
     unsigned int *att_cnt;        /* [n_layers * 8], zero at phase start */
 };
 
-/* ---- activation slices ---------------------------------------------------- */
+/* ---- activation vectors: memory -> LDS -> register slices ------------------- */
+
+/* Coherent 16-byte load (device scope: served past this XCD's L2). */
+__device__ __forceinline__ f32x4 vt_ldc4(const float *base, int idx4, int n_floats) {
+    __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, n_floats * 4, 0x00020000);
+    u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, idx4 * 16, 0, 16 /* sc1 */);
+    f32x4 f;
+    f.x = __uint_as_float(v.x); f.y = __uint_as_float(v.y);
+    f.z = __uint_as_float(v.z); f.w = __uint_as_float(v.w);
+    return f;
+}
+
+/* The whole workgroup copies n floats (n % 4 == 0) of a handed-over vector into LDS. */
+__device__ __forceinline__ void vt_stage(float *lds_x, const float *src, int n) {
+    f32x4 *dst = reinterpret_cast<f32x4 *>(lds_x);
+    for (int i = (int)threadIdx.x; i < n / 4; i += (int)blockDim.x) dst[i] = vt_ldc4(src, i, n);
+    __syncthreads();
+}
 
 template <int NK>
-__device__ __forceinline__ void vt_load_slice(f32x4 (&xa)[NK], f32x4 (&xb)[NK],
-                                              const float *x, int kofs) {
+__device__ __forceinline__ void vt_slice_lds(f32x4 (&xa)[NK], f32x4 (&xb)[NK], const float *lds_x, int kofs) {
+    const int lane = vt_lane();
+#pragma unroll
+    for (int c = 0; c < NK; c++) {
+        const f32x4 *p = reinterpret_cast<const f32x4 *>(lds_x + kofs + c * 512 + lane * 8);
+        xa[c] = p[0];
+        xb[c] = p[1];
+    }
+}
+
+template <int NK>
+__device__ __forceinline__ void vt_slice_global(f32x4 (&xa)[NK], f32x4 (&xb)[NK], const float *x, int kofs) {
     const int lane = vt_lane();
 #pragma unroll
     for (int c = 0; c < NK; c++) {
@@ -67,11 +104,13 @@ __device__ __forceinline__ void vt_load_slice(f32x4 (&xa)[NK], f32x4 (&xb)[NK],
     }
 }
 
-/* RMSNorm of the full 3072-vector, every wave for itself (NK = 6 covers it):
+/* RMSNorm of the staged 3072-vector, every wave for itself (NK = 6 covers it):
  * out = (x * 1/sqrt(mean(x^2)+eps)) * w  (voxtral_tts_kernels.c:333-349). */
 __device__ __forceinline__ void vt_rmsnorm_slice(f32x4 (&xa)[6], f32x4 (&xb)[6],
-                                                 const float *x, const float *w) {
-    vt_load_slice<6>(xa, xb, x, 0);
+                                                 const float *lds_x, const float *w) {
+    f32x4 wa[6], wb[6];
+    vt_slice_global<6>(wa, wb, w, 0);
+    vt_slice_lds<6>(xa, xb, lds_x, 0);
     float ss = 0.f;
 #pragma unroll
     for (int c = 0; c < 6; c++) {
@@ -81,19 +120,11 @@ __device__ __forceinline__ void vt_rmsnorm_slice(f32x4 (&xa)[6], f32x4 (&xb)[6],
         ss = fmaf(xb[c].z, xb[c].z, ss); ss = fmaf(xb[c].w, xb[c].w, ss);
     }
     ss = vt_wave_sum(ss);
-    const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(ss, (float)VT_DIM), VT_EPS)));
-    f32x4 wa[6], wb[6];
-    vt_load_slice<6>(wa, wb, w, 0);
+    const float inv = 1.0f / sqrtf(ss / (float)VT_DIM + VT_EPS);
 #pragma unroll
     for (int c = 0; c < 6; c++) {
-        xa[c].x = __fmul_rn(__fmul_rn(xa[c].x, inv), wa[c].x);
-        xa[c].y = __fmul_rn(__fmul_rn(xa[c].y, inv), wa[c].y);
-        xa[c].z = __fmul_rn(__fmul_rn(xa[c].z, inv), wa[c].z);
-        xa[c].w = __fmul_rn(__fmul_rn(xa[c].w, inv), wa[c].w);
-        xb[c].x = __fmul_rn(__fmul_rn(xb[c].x, inv), wb[c].x);
-        xb[c].y = __fmul_rn(__fmul_rn(xb[c].y, inv), wb[c].y);
-        xb[c].z = __fmul_rn(__fmul_rn(xb[c].z, inv), wb[c].z);
-        xb[c].w = __fmul_rn(__fmul_rn(xb[c].w, inv), wb[c].w);
+        xa[c] = (xa[c] * inv) * wa[c];
+        xb[c] = (xb[c] * inv) * wb[c];
     }
 }
 
@@ -194,9 +225,11 @@ __device__ __forceinline__ void vt_qkv_body(u32x4 (&ring)[VT_RING], const vt_lay
                                             const vt_step_args &a, int layer,
                                             const float *x_in, float *lds) {
     const vt_rows r = vt_qkv_rows();
+    float *lds_y = lds + VT_LDS_X;
+    vt_stage(lds, x_in, VT_DIM);
     f32x4 xa[6], xb[6];
-    vt_rmsnorm_slice(xa, xb, x_in, L.attn_norm);
-    vt_ring_run<6, 3>(ring, L.wqkv, VT_DIM, r, xa, xb, lds);
+    vt_rmsnorm_slice(xa, xb, lds, L.attn_norm);
+    vt_ring_run<6, 3>(ring, L.wqkv, VT_DIM, r, xa, xb, lds_y);
     __syncthreads();
     /* RoPE on adjacent pairs (voxtral_tts_kernels.c:616-634), then q to its
      * buffer and k, v straight into row `pos` of the cache. */
@@ -204,29 +237,42 @@ __device__ __forceinline__ void vt_qkv_body(u32x4 (&ring)[VT_RING], const vt_lay
     const size_t kv_row = ((size_t)(a.first_layer + layer) * a.kv_max + a.pos) * VT_KV_DIM;
     for (int t = (int)threadIdx.x; t < r.wg_nrows / 2; t += (int)blockDim.x) {
         const int g = r.wg_row0 + 2 * t;
-        const float v0 = lds[2 * t], v1 = lds[2 * t + 1];
+        const float v0 = lds_y[2 * t], v1 = lds_y[2 * t + 1];
         if (g < VT_Q_DIM + VT_KV_DIM) {
             const int d = (g & (VT_HEAD_DIM - 1)) >> 1;
             const float c = cs[2 * d], s = cs[2 * d + 1];
-            const float o0 = __fsub_rn(__fmul_rn(v0, c), __fmul_rn(v1, s));
-            const float o1 = __fadd_rn(__fmul_rn(v0, s), __fmul_rn(v1, c));
+            const float o0 = v0 * c - v1 * s;
+            const float o1 = v0 * s + v1 * c;
             float *dst = g < VT_Q_DIM ? a.q + g : a.kv_k + kv_row + (g - VT_Q_DIM);
-            dst[0] = o0;
-            dst[1] = o1;
+            vt_stc(dst, o0);
+            vt_stc(dst + 1, o1);
         } else {
             float *dst = a.kv_v + kv_row + (g - VT_Q_DIM - VT_KV_DIM);
-            dst[0] = v0;
-            dst[1] = v1;
+            vt_stc(dst, v0);
+            vt_stc(dst + 1, v1);
         }
     }
 }
 
 /* ---- phase 2: GQA attention of one query over the cache ------------------- */
-/* Workgroup = (kv head, chunk of positions).  A wave walks its positions;
- * lanes 16g..16g+15 serve query head 4*kvh+g and own 8 of the 128 dims.
- * Partials (max, sum, o[128]) are merged over the waves in LDS, written per
- * chunk, and the last workgroup to finish a kv head merges its chunks and
- * normalises (online-softmax algebra of voxtral_tts_kernels.c:426-462). */
+/* Workgroup = (kv head, chunk of positions); chunks hold at least
+ * VT_ATT_MIN_CHUNK positions, so short caches use one workgroup per kv head
+ * and need no cross-workgroup merge.  A wave walks its positions four at a
+ * time (all K and V rows of a batch are requested before any is used); lanes
+ * 16g..16g+15 serve query head 4*kvh+g and own 8 of the 128 dims.  Partials
+ * (max, sum, o[128]) are merged over the waves in LDS; with several chunks
+ * they are written per chunk and the last workgroup to finish a kv head
+ * merges them and normalises (online-softmax algebra of
+ * voxtral_tts_kernels.c:426-462). */
+__device__ __forceinline__ void vt_attn_geometry(int n, int nch_max, int nw, int &cs, int &nch) {
+    nch = (n + VT_ATT_MIN_CHUNK - 1) / VT_ATT_MIN_CHUNK;
+    if (nch > nch_max) nch = nch_max;
+    if (nch < 1) nch = 1;
+    cs = (n + nch - 1) / nch;
+    cs = (cs + nw - 1) / nw * nw;
+    nch = (n + cs - 1) / cs;
+}
+
 __device__ __forceinline__ void vt_attn_phase(const vt_step_args &a, int layer, float *lds) {
     const int G = (int)gridDim.x;
     const int nch_max = G / VT_KV_HEADS;
@@ -235,39 +281,48 @@ __device__ __forceinline__ void vt_attn_phase(const vt_step_args &a, int layer, 
     const int kvh = wg % VT_KV_HEADS, chunk = wg / VT_KV_HEADS;
     const int nw = (int)(blockDim.x >> 6), wave = vt_wave(), lane = vt_lane();
     const int n = a.pos + 1;
-    int cs = (n + nch_max - 1) / nch_max;
-    cs = (cs + nw - 1) / nw * nw;
-    const int nch = (n + cs - 1) / cs;
+    int cs, nch;
+    vt_attn_geometry(n, nch_max, nw, cs, nch);
     if (chunk >= nch) return;
     const int j0 = chunk * cs, j1 = min(n, j0 + cs);
 
     const int grp = lane >> 4, sub = lane & 15;
     const int head = kvh * 4 + grp;
-    const float scale = __fdiv_rn(1.0f, __fsqrt_rn((float)VT_HEAD_DIM));
-    const f32x4 *qp = reinterpret_cast<const f32x4 *>(a.q + head * VT_HEAD_DIM + sub * 8);
-    const f32x4 qa = qp[0], qb = qp[1];
+    const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
+    const f32x4 qa = vt_ldc4(a.q, (head * VT_HEAD_DIM + sub * 8) / 4, VT_Q_DIM);
+    const f32x4 qb = vt_ldc4(a.q, (head * VT_HEAD_DIM + sub * 8) / 4 + 1, VT_Q_DIM);
     const size_t layer_base = (size_t)(a.first_layer + layer) * a.kv_max * VT_KV_DIM;
     const float *kbase = a.kv_k + layer_base + kvh * VT_HEAD_DIM + sub * 8;
     const float *vbase = a.kv_v + layer_base + kvh * VT_HEAD_DIM + sub * 8;
 
     float m = -1e30f, l = 0.f;
     f32x4 oa = {0.f, 0.f, 0.f, 0.f}, ob = {0.f, 0.f, 0.f, 0.f};
-    for (int j = j0 + wave; j < j1; j += nw) {
-        const f32x4 *kp = reinterpret_cast<const f32x4 *>(kbase + (size_t)j * VT_KV_DIM);
-        const f32x4 *vp = reinterpret_cast<const f32x4 *>(vbase + (size_t)j * VT_KV_DIM);
-        const f32x4 ka = kp[0], kb = kp[1];
-        const f32x4 va = vp[0], vb = vp[1];
-        float s = qa.x * ka.x;
-        s = fmaf(qa.y, ka.y, s); s = fmaf(qa.z, ka.z, s); s = fmaf(qa.w, ka.w, s);
-        s = fmaf(qb.x, kb.x, s); s = fmaf(qb.y, kb.y, s); s = fmaf(qb.z, kb.z, s);
-        s = fmaf(qb.w, kb.w, s);
-        s = __fmul_rn(vt_row16_sum(s), scale);
-        const float mn = fmaxf(m, s);
-        const float corr = expf(m - mn), p = expf(s - mn);
-        l = fmaf(l, corr, p);
-        oa = oa * corr + va * p;
-        ob = ob * corr + vb * p;
-        m = mn;
+    for (int jb = j0 + wave; jb < j1; jb += 4 * nw) {
+        f32x4 ka[4], kb[4], va[4], vb[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int j = min(jb + u * nw, j1 - 1);        /* clamped rows are loaded but not used */
+            const f32x4 *kp = reinterpret_cast<const f32x4 *>(kbase + (size_t)j * VT_KV_DIM);
+            const f32x4 *vp = reinterpret_cast<const f32x4 *>(vbase + (size_t)j * VT_KV_DIM);
+            ka[u] = kp[0]; kb[u] = kp[1];
+            va[u] = vp[0]; vb[u] = vp[1];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            if (jb + u * nw < j1) {
+                float s = qa.x * ka[u].x;
+                s = fmaf(qa.y, ka[u].y, s); s = fmaf(qa.z, ka[u].z, s); s = fmaf(qa.w, ka[u].w, s);
+                s = fmaf(qb.x, kb[u].x, s); s = fmaf(qb.y, kb[u].y, s); s = fmaf(qb.z, kb[u].z, s);
+                s = fmaf(qb.w, kb[u].w, s);
+                s = vt_row16_sum(s) * scale;
+                const float mn = fmaxf(m, s);
+                const float corr = expf(m - mn), p = expf(s - mn);
+                l = fmaf(l, corr, p);
+                oa = oa * corr + va[u] * p;
+                ob = ob * corr + vb[u] * p;
+                m = mn;
+            }
+        }
     }
     /* merge the waves of this workgroup */
     float *part = lds;                                   /* [nw][4][VT_ATT_STRIDE] */
@@ -287,34 +342,54 @@ __device__ __forceinline__ void vt_attn_phase(const vt_step_args &a, int layer, 
             Ls = fmaf(pw[1], e, Ls);
             O = fmaf(pw[4 + d], e, O);
         }
-        float *dst = a.att_part + ((size_t)(kvh * 4 + g) * nch_max + chunk) * VT_ATT_STRIDE;
-        if (d == 0) { dst[0] = M; dst[1] = Ls; }
-        dst[4 + d] = O;
+        if (nch == 1) {
+            vt_stc(a.attn + (kvh * 4 + g) * VT_HEAD_DIM + d, O * (1.0f / Ls));
+        } else {
+            float *dst = a.att_part + ((size_t)(kvh * 4 + g) * nch_max + chunk) * VT_ATT_STRIDE;
+            if (d == 0) { vt_stc(dst, M); vt_stc(dst + 1, Ls); }
+            vt_stc(dst + 4 + d, O);
+        }
     }
+    if (nch == 1) return;
     /* last workgroup of this kv head merges the chunks */
     __shared__ int s_last;
-    __threadfence();
+    __builtin_amdgcn_s_waitcnt(0x0F70);                  /* partial stores acknowledged */
     __syncthreads();
     if (threadIdx.x == 0) {
         const unsigned old = __hip_atomic_fetch_add(a.att_cnt + layer * VT_KV_HEADS + kvh, 1u,
                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = (old == (unsigned)(nch - 1));
-        if (s_last) __threadfence();
     }
     __syncthreads();
     if (!s_last) return;
+    float *ml = lds;                                      /* [4][nch][2] staged (max, sum) pairs */
+    for (int t = (int)threadIdx.x; t < 4 * nch; t += (int)blockDim.x) {
+        const int g = t / nch, c = t % nch;
+        const float *src = a.att_part + ((size_t)(kvh * 4 + g) * nch_max + c) * VT_ATT_STRIDE;
+        ml[2 * t] = vt_ldc(src);
+        ml[2 * t + 1] = vt_ldc(src + 1);
+    }
+    __syncthreads();
     for (int t = (int)threadIdx.x; t < 4 * VT_HEAD_DIM; t += (int)blockDim.x) {
         const int g = t >> 7, d = t & 127;
-        const float *src = a.att_part + (size_t)(kvh * 4 + g) * nch_max * VT_ATT_STRIDE;
+        const float *src = a.att_part + (size_t)(kvh * 4 + g) * nch_max * VT_ATT_STRIDE + 4 + d;
         float M = -1e30f;
-        for (int c = 0; c < nch; c++) M = fmaxf(M, vt_ld_coherent(src + c * VT_ATT_STRIDE));
+        for (int c = 0; c < nch; c++) M = fmaxf(M, ml[2 * (g * nch + c)]);
         float Ls = 0.f, O = 0.f;
-        for (int c = 0; c < nch; c++) {
-            const float e = expf(vt_ld_coherent(src + c * VT_ATT_STRIDE) - M);
-            Ls = fmaf(vt_ld_coherent(src + c * VT_ATT_STRIDE + 1), e, Ls);
-            O = fmaf(vt_ld_coherent(src + c * VT_ATT_STRIDE + 4 + d), e, O);
+        for (int c0 = 0; c0 < nch; c0 += 4) {
+            float o[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) o[u] = vt_ldc(src + (size_t)min(c0 + u, nch - 1) * VT_ATT_STRIDE);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (c0 + u < nch) {
+                    const float e = expf(ml[2 * (g * nch + c0 + u)] - M);
+                    Ls = fmaf(ml[2 * (g * nch + c0 + u) + 1], e, Ls);
+                    O = fmaf(o[u], e, O);
+                }
+            }
         }
-        a.attn[(kvh * 4 + g) * VT_HEAD_DIM + d] = __fmul_rn(O, __fdiv_rn(1.0f, Ls));
+        vt_stc(a.attn + (kvh * 4 + g) * VT_HEAD_DIM + d, O * (1.0f / Ls));
     }
 }
 
@@ -329,13 +404,15 @@ __device__ __forceinline__ void vt_wo_prefetch(u32x4 (&ring)[VT_RING], const vt_
 __device__ __forceinline__ void vt_wo_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
                                            const vt_step_args &a, const float *x_in, float *lds) {
     const vt_rows r = vt_wo_rows();
+    float *lds_y = lds + VT_LDS_X;
+    vt_stage(lds, a.attn, VT_Q_DIM);
     f32x4 xa[4], xb[4];
-    vt_load_slice<4>(xa, xb, a.attn, r.kofs);
-    vt_ring_run<4, 4>(ring, L.wo, VT_Q_DIM, r, xa, xb, lds);
+    vt_slice_lds<4>(xa, xb, lds, r.kofs);
+    vt_ring_run<4, 4>(ring, L.wo, VT_Q_DIM, r, xa, xb, lds_y);
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows; t += (int)blockDim.x) {
-        const float y = __fadd_rn(lds[t], lds[r.wg_nrows + t]);
-        a.x[r.wg_row0 + t] = __fadd_rn(x_in[r.wg_row0 + t], y);
+        const float y = lds_y[t] + lds_y[r.wg_nrows + t];
+        vt_stc(a.x + r.wg_row0 + t, vt_ldc(x_in + r.wg_row0 + t) + y);
     }
 }
 
@@ -350,14 +427,16 @@ __device__ __forceinline__ void vt_w13_prefetch(u32x4 (&ring)[VT_RING], const vt
 __device__ __forceinline__ void vt_w13_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
                                             const vt_step_args &a, float *lds) {
     const vt_rows r = vt_w13_rows();
+    float *lds_y = lds + VT_LDS_X;
+    vt_stage(lds, a.x, VT_DIM);
     f32x4 xa[6], xb[6];
-    vt_rmsnorm_slice(xa, xb, a.x, L.ffn_norm);
-    vt_ring_run<6, 3>(ring, L.w13, VT_DIM, r, xa, xb, lds);
+    vt_rmsnorm_slice(xa, xb, lds, L.ffn_norm);
+    vt_ring_run<6, 3>(ring, L.w13, VT_DIM, r, xa, xb, lds_y);
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows / 2; t += (int)blockDim.x) {
-        const float g = lds[2 * t], u = lds[2 * t + 1];
-        const float sg = __fdiv_rn(g, __fadd_rn(1.0f, expf(-g)));     /* voxtral_tts_kernels.c:361-366 */
-        a.h[r.wg_row0 / 2 + t] = __fmul_rn(sg, u);
+        const float g = lds_y[2 * t], u = lds_y[2 * t + 1];
+        const float sg = g / (1.0f + expf(-g));                      /* voxtral_tts_kernels.c:361-366 */
+        vt_stc(a.h + r.wg_row0 / 2 + t, sg * u);
     }
 }
 
@@ -372,30 +451,38 @@ __device__ __forceinline__ void vt_w2_prefetch(u32x4 (&ring)[VT_RING], const vt_
 __device__ __forceinline__ void vt_w2_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
                                            const vt_step_args &a, float *lds) {
     const vt_rows r = vt_w2_rows();
+    float *lds_y = lds + VT_LDS_X;
+    vt_stage(lds, a.h, VT_FFN);
     f32x4 xa[9], xb[9];
-    vt_load_slice<9>(xa, xb, a.h, r.kofs);
-    vt_ring_run<9, 2>(ring, L.w2, VT_FFN, r, xa, xb, lds);
+    vt_slice_lds<9>(xa, xb, lds, r.kofs);
+    vt_ring_run<9, 2>(ring, L.w2, VT_FFN, r, xa, xb, lds_y);
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows; t += (int)blockDim.x) {
-        const float y = __fadd_rn(lds[t], lds[r.wg_nrows + t]);
-        a.x[r.wg_row0 + t] = __fadd_rn(a.x[r.wg_row0 + t], y);
+        const float y = lds_y[t] + lds_y[r.wg_nrows + t];
+        vt_stc(a.x + r.wg_row0 + t, vt_ldc(a.x + r.wg_row0 + t) + y);
     }
 }
 
-/* ---- final RMSNorm (one workgroup) ----------------------------------------- */
+/* ---- RMSNorm of one row by one workgroup ------------------------------------ */
 
+template <bool COHERENT>
 __device__ __forceinline__ void vt_block_rmsnorm(float *out, const float *x, const float *w,
                                                  int dim, float eps, float *lds) {
     float ss = 0.f;
-    for (int i = (int)threadIdx.x; i < dim; i += (int)blockDim.x) ss = fmaf(x[i], x[i], ss);
+    for (int i = (int)threadIdx.x; i < dim; i += (int)blockDim.x) {
+        const float v = COHERENT ? vt_ldc(x + i) : x[i];
+        ss = fmaf(v, v, ss);
+    }
     ss = vt_wave_sum(ss);
     if (vt_lane() == 0) lds[vt_wave()] = ss;
     __syncthreads();
     float tot = 0.f;
     for (int w_ = 0; w_ < (int)(blockDim.x >> 6); w_++) tot += lds[w_];
-    const float inv = __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(tot, (float)dim), eps)));
-    for (int i = (int)threadIdx.x; i < dim; i += (int)blockDim.x)
-        out[i] = __fmul_rn(__fmul_rn(x[i], inv), w[i]);
+    const float inv = 1.0f / sqrtf(tot / (float)dim + eps);
+    for (int i = (int)threadIdx.x; i < dim; i += (int)blockDim.x) {
+        const float v = COHERENT ? vt_ldc(x + i) : x[i];
+        out[i] = (v * inv) * w[i];
+    }
     __syncthreads();
 }
 

@@ -90,47 +90,74 @@ __device__ __forceinline__ float vt_dot8(u32x4 w, f32x4 xa, f32x4 xb, float acc)
     return acc;
 }
 
-/* Coherent (device-scope) scalar accesses for data exchanged between
- * workgroups inside one kernel. */
-__device__ __forceinline__ float vt_ld_coherent(const float *p) {
+/* Device-scope coherent accesses for the small vectors that workgroups hand
+ * to each other inside one kernel.  Each XCD has its own L2, so such data is
+ * written through to memory and read past the L2 (relaxed agent-scope
+ * atomics); no cache-wide write-back or invalidate is ever issued. */
+__device__ __forceinline__ float vt_ldc(const float *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void vt_stc(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned vt_ldc_u32(const unsigned *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void vt_stc_u32(unsigned *p, unsigned v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
-/* ---- bounded grid barrier -------------------------------------------------
- * All workgroups of a persistent kernel are co-resident (the launch is
- * cooperative and sized to the device).  `counter` only grows: barrier number
- * b of a launch is passed once the counter reaches base + (b+1)*gridDim.x.
- * The spin is bounded by a wall-clock budget; on expiry (or when another
- * workgroup has raised `abort_flag`) the barrier returns false and the caller
- * leaves the kernel, so every wave always reaches the end of the grid. */
+/* ---- bounded grid barrier over per-workgroup flags -------------------------
+ * All workgroups of a persistent kernel are co-resident (the grid is sized to
+ * the device, one workgroup per CU).  Workgroup w announces barrier number e
+ * by writing e to flags[w]; the first wave of every workgroup polls all flags
+ * (one coherent load per lane and 64 flags) until each has reached e.  No
+ * read-modify-write is involved, so arrivals do not serialise.  Epochs only
+ * grow, across launches too (the host passes the first epoch of a launch).
+ * The spin is bounded by a wall-clock budget; on expiry, or when another
+ * workgroup has raised `abort_flag`, the barrier returns false and the caller
+ * leaves the kernel, so every wave always reaches the end of the grid.
+ *
+ * Data handed over a barrier must be written with vt_stc and read with
+ * vt_ldc: __syncthreads() makes every wave wait for its own stores to be
+ * acknowledged before the flag is written. */
 struct vt_grid_sync {
-    unsigned long long *counter;
+    unsigned *flags;                /* [gridDim.x] */
     int *abort_flag;
-    unsigned long long target;      /* value that releases the next barrier */
+    unsigned epoch;                 /* epoch of the next barrier */
     unsigned long long timeout;     /* wall_clock64 ticks (100 MHz) */
 };
 
-__device__ __forceinline__ bool vt_grid_barrier(vt_grid_sync &gs, int *lds_flag) {
+__device__ __forceinline__ void vt_barrier_arrive(vt_grid_sync &gs) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);          /* vmcnt(0): this wave's stores are acknowledged */
     __syncthreads();
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0) vt_stc_u32(gs.flags + blockIdx.x, gs.epoch);
+}
+
+__device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag) {
+    if (threadIdx.x < VT_WAVE) {
+        const int G = (int)gridDim.x;
+        const unsigned long long t0 = wall_clock64();
         int ok = 1;
-        __threadfence();                                   /* release this workgroup's stores */
-        __hip_atomic_fetch_add(gs.counter, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        unsigned long long t0 = wall_clock64();
-        while (__hip_atomic_load(gs.counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < gs.target) {
-            __builtin_amdgcn_s_sleep(2);
+        for (;;) {
+            int done = 1;
+            for (int i = (int)threadIdx.x; i < G; i += VT_WAVE)
+                done &= (int)(vt_ldc_u32(gs.flags + i) - gs.epoch) >= 0;
+            if (__all(done)) break;
             if (__hip_atomic_load(gs.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
                 wall_clock64() - t0 > gs.timeout) {
-                __hip_atomic_store(gs.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 ok = 0;
                 break;
             }
         }
-        __threadfence();                                   /* acquire the other workgroups' stores */
-        *lds_flag = ok;
+        ok = __all(ok);
+        if (threadIdx.x == 0) {
+            if (!ok) __hip_atomic_store(gs.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *lds_flag = ok;
+        }
     }
     __syncthreads();
-    gs.target += gridDim.x;
+    gs.epoch += 1u;
     return *lds_flag != 0;
 }
 

@@ -117,7 +117,7 @@ done:
 __global__ void __launch_bounds__(256)
 vt_rms_norm_kernel(float *out, const float *x, const float *w, int dim, float eps) {
     __shared__ float lds[VT_MAX_WAVES];
-    vt_block_rmsnorm(out + (size_t)blockIdx.x * dim, x + (size_t)blockIdx.x * dim, w, dim, eps, lds);
+    vt_block_rmsnorm<false>(out + (size_t)blockIdx.x * dim, x + (size_t)blockIdx.x * dim, w, dim, eps, lds);
 }
 
 void vt_launch_rms_norm(float *d_out, const float *d_x, const float *d_w, int seq, int dim, float eps) {

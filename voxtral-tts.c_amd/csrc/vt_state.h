@@ -15,7 +15,6 @@
 
 #define VT_MAX_WAVES 8
 #define VT_STEP_THREADS 512
-#define VT_ATT_LDS_FLOATS (VT_MAX_WAVES * 4 * VT_ATT_STRIDE)
 #define VT_AC_SEQ 3
 #define VT_AC_DIM_IN 36
 #define VT_SEM_PADDED 8320
@@ -58,8 +57,8 @@ struct vt_state {
     /* decode work buffers */
     float *d_x, *d_q, *d_attn, *d_h, *d_att_part, *d_embed, *d_hidden;
     unsigned int *d_att_cnt;
-    unsigned long long *d_bar_counter;
-    unsigned long long bar_base;
+    unsigned int *d_bar_flags;    /* one flag per workgroup of the persistent kernel */
+    unsigned int bar_epoch;       /* last barrier epoch handed to a launch */
     int *d_abort;
     float *h_pin;                 /* pinned staging: [3072 in][3072 out + flag] */
 
