@@ -107,6 +107,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--mode", type=int, default=0, help="0 persistent kernel, 1 per-phase kernels")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch one plain elementwise kernel (vt_add_kernel, a += b over 64 Mi floats: "
+                         "512 MiB read, 256 MiB written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                         "can be scaled by a kernel of known traffic")
     ap.add_argument("--traffic-kib", type=float, default=None,
                     help="HBM bytes per launch measured with rocprofv3 --pmc (KiB), if known")
     args = ap.parse_args()
@@ -133,6 +137,16 @@ def main():
     hip.upload_decoder(layers, final_norm, N_LAYERS)
     d_proj = H.DevBuf.from_numpy(lib, proj)
     t_up = time.time() - t0
+
+    if args.calibrate:
+        n_cal = 64 << 20
+        ca, cb = H.DevBuf(lib, 4 * n_cal), H.DevBuf(lib, 4 * n_cal)
+        lib.tts_hip_memset(ca.ptr, 0, 4 * n_cal)
+        lib.tts_hip_memset(cb.ptr, 0, 4 * n_cal)
+        lib.tts_hip_add_inplace(ca.ptr, cb.ptr, n_cal)
+        lib.tts_hip_sync()
+        ca.free()
+        cb.free()
 
     # prefill the prompt on the GPU; the first decode input is the last residual row
     # pushed through the feedback projection (any O(1) vector would do)

@@ -126,3 +126,9 @@ void ref_audio_embed_set(tts_ctx_t *ctx, uint16_t *emb) {
 void ref_audio_embed_forward(tts_ctx_t *ctx, const int *codes, float *out) {
     tts_audio_embed_forward(ctx, codes, out);
 }
+
+/* Addresses of the weight structs inside the context: what the reference's
+ * tts_load passes to the upload entry points (voxtral_tts.c:96-99). */
+void *ref_decoder_ptr(tts_ctx_t *ctx) { return &ctx->decoder; }
+void *ref_acoustic_ptr(tts_ctx_t *ctx) { return &ctx->acoustic; }
+int ref_kv_max(tts_ctx_t *ctx) { return ctx->kv_cache_max; }

@@ -14,7 +14,8 @@ import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-LIB_PATH = os.path.join(CSRC, "libvoxtral_tts_hip.so")
+# VOXTRAL_TTS_HIP_LIB selects another build of the same library (e.g. an instrumented one).
+LIB_PATH = os.environ.get("VOXTRAL_TTS_HIP_LIB") or os.path.join(CSRC, "libvoxtral_tts_hip.so")
 
 DEC_LAYERS = 26
 AC_LAYERS = 3

@@ -19,11 +19,30 @@
 
 /* Arrive at the grid barrier, request the next phase's first weight rows while
  * the other workgroups arrive, then wait. */
+#ifdef VT_TRACE
+/* Build-time instrumentation (never in the shipped library): workgroups 0 and
+ * gridDim.x-1 record the 100 MHz wall clock at the points of every phase. */
+__device__ unsigned long long vt_trace_buf[2 * 4096];
+__device__ __forceinline__ void vt_tr(int &n) {
+    if (threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == gridDim.x - 1) && n < 4096)
+        vt_trace_buf[(blockIdx.x ? 4096 : 0) + n] = wall_clock64();
+    n++;
+}
+#define VT_TR(n) vt_tr(n)
+#else
+#define VT_TR(n) ((void)0)
+#endif
+
 template <class F>
-__device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between) {
+__device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between, int &tn) {
+    VT_TR(tn);                      /* body done */
     vt_barrier_arrive(gs);
+    VT_TR(tn);                      /* arrived */
     between();
-    return vt_barrier_wait(gs, flag);
+    VT_TR(tn);                      /* prefetch requested */
+    const bool ok = vt_barrier_wait(gs, flag);
+    VT_TR(tn);                      /* released */
+    return ok;
 }
 
 __global__ void __launch_bounds__(VT_STEP_THREADS)
@@ -31,6 +50,7 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
     __shared__ __attribute__((aligned(16))) float lds[VT_LDS_FLOATS];
     __shared__ int s_flag;
     u32x4 ring[VT_RING];
+    int tn = 0;
 
     if (blockIdx.x == 0)
         for (int t = (int)threadIdx.x; t < a.n_layers * VT_KV_HEADS; t += (int)blockDim.x)
@@ -41,16 +61,16 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
     for (int l = 0; l < a.n_layers; l++) {
         const vt_layer_dev L = a.layers[l];
         vt_qkv_body(ring, L, a, l, x_in, lds);
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_wo_prefetch(ring, L); })) return;
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_wo_prefetch(ring, L); }, tn)) return;
         vt_attn_phase(a, l, lds);
-        if (!vt_barrier_then(gs, &s_flag, [] {})) return;
+        if (!vt_barrier_then(gs, &s_flag, [] {}, tn)) return;
         vt_wo_body(ring, L, a, x_in, lds);
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L); })) return;
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L); }, tn)) return;
         vt_w13_body(ring, L, a, lds);
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w2_prefetch(ring, L); })) return;
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w2_prefetch(ring, L); }, tn)) return;
         vt_w2_body(ring, L, a, lds);
         const bool more = l + 1 < a.n_layers;
-        if (!vt_barrier_then(gs, &s_flag, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1]); }))
+        if (!vt_barrier_then(gs, &s_flag, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1]); }, tn))
             return;
         x_in = a.x;
     }
@@ -203,6 +223,13 @@ static int step_aborted(int flag) {
     g_vt.bar_epoch = 0;
     return -1;
 }
+
+#ifdef VT_TRACE
+extern "C" void tts_hip_trace_read(unsigned long long *out) {
+    (void)hipDeviceSynchronize();
+    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(vt_trace_buf), sizeof(unsigned long long) * 2 * 4096);
+}
+#endif
 
 extern "C" void tts_hip_llm_forward_device(float *d_out_hidden, const float *d_input_embed, int pos) {
     if (g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_llm_forward: no weights uploaded"); return; }
