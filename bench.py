@@ -105,7 +105,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--mode", type=int, default=0, help="0 persistent kernel, 1 per-phase kernels")
+    ap.add_argument("--mode", type=int, default=0, help="0 persistent kernel, 1 per-phase kernels, 2 streaming kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one plain elementwise kernel (vt_add_kernel, a += b over 64 Mi floats: "
@@ -221,14 +221,14 @@ def main():
                         "hidden fed back through a 3072x3072 bf16 projection (BASELINE.json configs[2])",
             "layers": N_LAYERS, "prompt": PROMPT, "positions": [pos0, pos0 + K - 1],
             "weights": "bf16 N(0,0.02) seeded, truncated", "activations": "f32",
-            "schedule": "persistent whole-step kernel" if args.mode == 0 else "one kernel per phase",
+            "schedule": ("persistent whole-step kernel", "one kernel per phase", "streaming whole-step kernel")[args.mode],
         },
         "frames_per_s": round(1000.0 / ms_step, 1),
         "hbm_gbps": round((bytes_launch + 2 * S.DIM * S.DIM) / (ms_step * 1e-3) / 1e9, 1),
         "hbm_frac_of_peak": round((bytes_launch + 2 * S.DIM * S.DIM) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "ms_per_frame_normalised_6p8GB": round(ms_kernel * 6.8e9 / bytes_launch, 4),
         "roofline": {
-            "kernel": "vt_decode_step_kernel" if args.mode == 0 else "5 phase kernels per layer",
+            "kernel": ("vt_decode_step_kernel", "5 phase kernels per layer", "vt_decode_stream_kernel")[args.mode],
             "bound": "hbm",
             "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),

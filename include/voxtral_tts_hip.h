@@ -192,7 +192,8 @@ void tts_hip_predict_velocity_cfg(float *out_v_cond, float *out_v_uncond, const 
 void tts_hip_acoustic_frame(int *out_codes, const float *llm_hidden, const float *x0,
                             float *out_x);
 
-/* 0 = persistent whole-step kernel (default), 1 = one kernel per phase. */
+/* Decode schedule: 0 = persistent whole-step kernel (default), 1 = one kernel per
+ * phase, 2 = streaming whole-step kernel (256-CU devices; experimental). */
 void tts_hip_set_decode_mode(int mode);
 /* Number of failed calls since init, and the text of the last failure. */
 int tts_hip_error_count(void);

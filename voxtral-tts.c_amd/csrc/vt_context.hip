@@ -128,6 +128,7 @@ extern "C" int tts_hip_init(int kv_cache_max) {
         {(void **)&g_vt.d_hidden, sizeof(float) * (VT_DIM + 64)},
         {(void **)&g_vt.d_bar_flags, sizeof(unsigned) * (size_t)g_vt.grid + 256},
         {(void **)&g_vt.d_abort, 256},
+        {(void **)&g_vt.d_dummy, 4096},
     };
     for (size_t i = 0; i < sizeof bufs / sizeof bufs[0]; i++) {
         if (!(*bufs[i].p = vt_dev_alloc(bufs[i].bytes))) return -1;
@@ -160,7 +161,7 @@ extern "C" void tts_hip_free(void) {
                     g_vt.ac.time_inv_freq, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu,
                     g_vt.d_rope, g_vt.d_x, g_vt.d_q, g_vt.d_attn, g_vt.d_h, g_vt.d_att_part,
                     g_vt.d_att_cnt, g_vt.d_embed, g_vt.d_hidden, g_vt.d_bar_flags,
-                    g_vt.d_abort, g_vt.d_scratch};
+                    g_vt.d_abort, g_vt.d_dummy, g_vt.d_scratch};
     for (size_t i = 0; i < sizeof ptrs / sizeof ptrs[0]; i++)
         if (ptrs[i]) (void)hipFree(ptrs[i]);
     if (g_vt.h_pin) (void)hipHostFree(g_vt.h_pin);

@@ -10,6 +10,11 @@
  *           HBM stream does not stop while the tiny activation vectors are
  *           exchanged between workgroups.
  *   mode 1  one kernel per phase (5 launches per layer), same numerics.
+ *   mode 2  the streaming kernel of vt_decode_stream.hip (256-CU devices only):
+ *           weight streaming decoupled from synchronisation, 6 stream waves + 1
+ *           control wave per CU.  Correct and reproducible, but not yet faster
+ *           than mode 0 (its control path pays the CU's shared memory queue on
+ *           every hand-over); opt-in.
  */
 #include "vt_state.h"
 
@@ -180,7 +185,10 @@ int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
 
     const dim3 grid(g_vt.grid), block(VT_STEP_THREADS);
     hipStream_t st = g_vt.stream;
-    if (g_vt.decode_mode == 0) {
+    if (g_vt.decode_mode == 2) {
+        if (!vt_stream_supported()) { vt_set_error("decode step: the streaming schedule needs a 256-CU device"); return -1; }
+        return vt_run_step_stream(a);
+    } else if (g_vt.decode_mode == 0) {
         vt_grid_sync gs;
         gs.flags = g_vt.d_bar_flags;
         gs.abort_flag = g_vt.d_abort;

@@ -37,8 +37,12 @@ __device__ __forceinline__ float vt_bf16_hi(unsigned int w) { return __uint_as_f
 /* 16-byte streaming load of 8 bf16 weights: weights are read once per step,
  * so they are marked non-temporal to keep the small activation vectors and
  * the KV cache resident in L2. */
+typedef __attribute__((address_space(1))) const u32x4 vt_global_u32x4;
 __device__ __forceinline__ u32x4 vt_ldw(const uint16_t *p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    /* weights live in device memory: say so, or pointers read from a struct in
+     * memory are treated as generic and become FLAT loads, which also occupy
+     * the LDS counter */
+    return __builtin_nontemporal_load((vt_global_u32x4 *)p);
 }
 
 template <int CTRL>
@@ -75,6 +79,16 @@ __device__ __forceinline__ float vt_wave_sum(float v) {
     float a = vt_readlane(v, 0) + vt_readlane(v, 16);
     float b = vt_readlane(v, 32) + vt_readlane(v, 48);
     return a + b;
+}
+
+/* Full wave64 sum that ends in lane 63 only (other lanes hold partial sums):
+ * 4 steps inside each row of 16, then row_bcast:15 into rows 1 and 3 and
+ * row_bcast:31 into rows 2 and 3.  No scalar round trip. */
+__device__ __forceinline__ float vt_wave_sum_lane63(float v) {
+    v = vt_row16_sum(v);
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xa, 0xf, false));
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xc, 0xf, false));
+    return v;
 }
 
 /* 8 weights (one 16-byte load) times 8 activations, accumulated with FMA. */

@@ -60,6 +60,7 @@ struct vt_state {
     unsigned int *d_bar_flags;    /* one flag per workgroup of the persistent kernel */
     unsigned int bar_epoch;       /* last barrier epoch handed to a launch */
     int *d_abort;
+    uint16_t *d_dummy;            /* small resident block requested in place of a layer beyond the last */
     float *h_pin;                 /* pinned staging: [3072 in][3072 out + flag] */
 
     /* generic scratch (prefill / acoustic / linear) */
@@ -88,6 +89,8 @@ void vt_launch_attention(float *d_out, const float *d_Q, const float *d_K, const
                          int seq_q, int q_offset, int seq_k, int causal, int n_heads,
                          int n_kv_heads, int head_dim, float scale, int kv_stride, int q_stride);
 void vt_launch_add(float *d_a, const float *d_b, int n);
+int vt_stream_supported(void);
+int vt_run_step_stream(const vt_step_args &a);
 int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
                 const float *d_final_norm, const float *d_in, float *d_out, int pos);
 
