@@ -104,6 +104,18 @@ __device__ __forceinline__ float vt_dot8(u32x4 w, f32x4 xa, f32x4 xb, float acc)
     return acc;
 }
 
+/* fp32 -> two bf16 planes: hi = bf16(x) (round to nearest even) and
+ * lo = bf16(x - hi); x - hi is exact in fp32, so hi + lo carries x to about
+ * 2^-17 relative.  Finite inputs only. */
+__device__ __forceinline__ unsigned vt_bf16_rne(float x) {
+    const unsigned u = __float_as_uint(x);
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ void vt_split_planes(float x, unsigned &hi, unsigned &lo) {
+    hi = vt_bf16_rne(x);
+    lo = vt_bf16_rne(__fsub_rn(x, __uint_as_float(hi << 16)));
+}
+
 /* Device-scope coherent accesses for the small vectors that workgroups hand
  * to each other inside one kernel.  Each XCD has its own L2, so such data is
  * written through to memory and read past the L2 (relaxed agent-scope

@@ -1,0 +1,262 @@
+/*
+ * vt_gemm.hip - bf16 MFMA matrix product for rows of activations (seq_len > 1):
+ * C[M,N] = X[M,K] * W[N,K]^T with fp32 accumulation, the sequence-level linear
+ * of the CPU path (tts_linear_nobias_bf16 with seq_len > 1,
+ * voxtral_tts_kernels.c:187-198, and the triple loop it falls to, :127-138).
+ *
+ * Weights are bf16 already.  The fp32 activations are carried as two bf16
+ * planes, hi = bf16(x) and lo = bf16(x - hi), so that hi + lo represents x to
+ * about 2^-17 relative; every weight tile is multiplied with both planes
+ * (two MFMAs per tile pair) and the sums land in the same fp32 accumulator.
+ * That keeps the result within a few fp32 ulps of the sequential CPU sum while
+ * all products run on the matrix cores.
+ *
+ * Tiling: workgroup tile 128 x 128, K step 64, four waves in a 2 x 2 grid of
+ * 64 x 64 wave tiles, v_mfma_f32_32x32x16_bf16.  Tiles are staged through LDS
+ * with a row pitch of 144 bytes (128 of data + 16 of padding): the 16 lanes of
+ * a 16-byte fragment read then cover all 64 banks once.  One LDS stage; the
+ * next K step is fetched into registers while the current one is multiplied,
+ * and two workgroups share a CU.  Workgroups that need the same weight tile
+ * (the M tiles of one N tile) get consecutive slots on one XCD, so the tile is
+ * fetched from HBM once and served from that XCD's L2 afterwards.  Long K can
+ * be cut into `splits` ranges that write separate partial planes; the caller
+ * adds them in a fixed order (vt_residual_norm_split_kernel).
+ */
+#include "vt_state.h"
+#include "vt_gemm.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(1))) const u32x4 vt_gptr_u32x4;
+
+#define GM_TILE 128
+#define GM_BK   64
+#define GM_ROWB 144
+#define GM_MAT  (GM_TILE * GM_ROWB)
+
+__device__ __forceinline__ u32x4 gm_ld(const uint16_t *p) { return *(vt_gptr_u32x4 *)p; }
+__device__ __forceinline__ bf16x8 gm_frag(const unsigned char *p) {
+    return __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(p));
+}
+
+__global__ void __launch_bounds__(256, 2)
+vt_gemm_mfma_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const uint16_t *W,
+                    int M, int N, int K, int k_split, int m_tiles, int n_tiles) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[3 * GM_MAT];
+    const int id = (int)blockIdx.x;
+    int mt, nt, sp;
+    if ((n_tiles & 7) == 0) {
+        /* slot id lands on XCD id % 8: keep the M tiles of one N tile there */
+        const int x = id & 7, q = id >> 3, r = q / m_tiles, npx = n_tiles >> 3;
+        mt = q % m_tiles;
+        nt = (r % npx) * 8 + x;
+        sp = r / npx;
+    } else {
+        const int r = id / m_tiles;
+        mt = id % m_tiles;
+        nt = r % n_tiles;
+        sp = r / n_tiles;
+    }
+    const int t = (int)threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int lr = t >> 3, lc = t & 7;               /* staging: row lr + 32 i, 16-byte chunk lc */
+    const int k0 = sp * k_split, tiles = k_split / GM_BK;
+
+    const uint16_t *pa[4], *pl[4], *pw[4];
+    bool live[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int gm = mt * GM_TILE + lr + 32 * i;
+        live[i] = gm < M;
+        const size_t ao = (size_t)(live[i] ? gm : 0) * K + k0 + lc * 8;
+        pa[i] = Ahi + ao;
+        pl[i] = Alo + ao;
+        pw[i] = W + (size_t)(nt * GM_TILE + lr + 32 * i) * K + k0 + lc * 8;
+    }
+
+    u32x4 ra[4], rl[4], rb[4];
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        ra[i] = live[i] ? gm_ld(pa[i]) : zero;
+        rl[i] = live[i] ? gm_ld(pl[i]) : zero;
+        rb[i] = gm_ld(pw[i]);
+    }
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
+
+    const int st_off = lr * GM_ROWB + lc * 16;
+    const int fa_off = (64 * wm + (lane & 31)) * GM_ROWB + (lane >> 5) * 16;
+    const int fb_off = (64 * wn + (lane & 31)) * GM_ROWB + (lane >> 5) * 16 + 2 * GM_MAT;
+
+    for (int kt = 0; kt < tiles; kt++) {
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            *reinterpret_cast<u32x4 *>(lds + st_off + 32 * i * GM_ROWB) = ra[i];
+            *reinterpret_cast<u32x4 *>(lds + GM_MAT + st_off + 32 * i * GM_ROWB) = rl[i];
+            *reinterpret_cast<u32x4 *>(lds + 2 * GM_MAT + st_off + 32 * i * GM_ROWB) = rb[i];
+        }
+        __syncthreads();
+        if (kt + 1 < tiles) {
+            const int adv = (kt + 1) * GM_BK;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                ra[i] = live[i] ? gm_ld(pa[i] + adv) : zero;
+                rl[i] = live[i] ? gm_ld(pl[i] + adv) : zero;
+                rb[i] = gm_ld(pw[i] + adv);
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < GM_BK / 16; ks++) {
+            bf16x8 fa[2], fl[2], fb[2];
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                fa[b] = gm_frag(lds + fa_off + 32 * b * GM_ROWB + ks * 32);
+                fl[b] = gm_frag(lds + GM_MAT + fa_off + 32 * b * GM_ROWB + ks * 32);
+                fb[b] = gm_frag(lds + fb_off + 32 * b * GM_ROWB + ks * 32);
+            }
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int b = 0; b < 2; b++) {
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fl[a], fb[b], acc[a][b], 0, 0, 0);
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fb[b], acc[a][b], 0, 0, 0);
+                }
+        }
+    }
+
+    /* accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 */
+    float *Cs = C + (size_t)sp * M * N;
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const int col = nt * GM_TILE + 64 * wn + 32 * b + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = mt * GM_TILE + 64 * wm + 32 * a + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (row < M) Cs[(size_t)row * N + col] = acc[a][b][v];
+            }
+        }
+}
+
+int vt_gemm_shape_ok(int M, int N, int K, int splits) {
+    return M >= 1 && splits >= 1 && N % GM_TILE == 0 && K % splits == 0 && (K / splits) % GM_BK == 0;
+}
+
+void vt_launch_gemm(float *d_C, const uint16_t *d_Ahi, const uint16_t *d_Alo, const uint16_t *d_W,
+                    int M, int N, int K, int splits) {
+    const int m_tiles = (M + GM_TILE - 1) / GM_TILE, n_tiles = N / GM_TILE;
+    hipLaunchKernelGGL(vt_gemm_mfma_kernel, dim3(m_tiles * n_tiles * splits), dim3(256), 0, g_vt.stream,
+                       d_C, d_Ahi, d_Alo, d_W, M, N, K, K / splits, m_tiles, n_tiles);
+}
+
+/* ---- fp32 -> (hi, lo) bf16 planes ---------------------------------------------- */
+
+__global__ void vt_split_kernel(uint16_t *hi, uint16_t *lo, const float *x, size_t n2) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n2;
+         i += (size_t)gridDim.x * blockDim.x) {
+        const f32x2 v = reinterpret_cast<const f32x2 *>(x)[i];
+        unsigned h0, l0, h1, l1;
+        vt_split_planes(v.x, h0, l0);
+        vt_split_planes(v.y, h1, l1);
+        reinterpret_cast<unsigned *>(hi)[i] = h0 | (h1 << 16);
+        reinterpret_cast<unsigned *>(lo)[i] = l0 | (l1 << 16);
+    }
+}
+
+static int gm_blocks(size_t n) { size_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : b); }
+
+void vt_launch_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_x, size_t n) {
+    hipLaunchKernelGGL(vt_split_kernel, dim3(gm_blocks(n / 2)), dim3(256), 0, g_vt.stream, d_hi, d_lo, d_x, n / 2);
+}
+
+/* One workgroup per row of 3072 floats (256 threads x 12):
+ *   x[row] += part[0][row] + part[1][row] + ...   (splits > 0; fixed order)
+ *   (hi, lo)[row] = split(rmsnorm(x[row]) * w)     (w != NULL)
+ * The residual add and the normalisation of voxtral_tts_llm.c:332-336,354 /
+ * :338-341 in one pass over the row. */
+__global__ void __launch_bounds__(256)
+vt_residual_norm_split_kernel(float *x, const float *part, int splits, size_t part_stride,
+                              const float *w, uint16_t *hi, uint16_t *lo, float eps) {
+    __shared__ float red[4];
+    const size_t row = blockIdx.x;
+    float v[VT_DIM / 256];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < VT_DIM / 256; j++) {
+        const size_t i = row * VT_DIM + threadIdx.x + 256 * j;
+        float a = x[i];
+        if (splits > 0) {
+            float p = part[i];
+            for (int s = 1; s < splits; s++) p = __fadd_rn(p, part[(size_t)s * part_stride + i]);
+            a = __fadd_rn(a, p);
+            x[i] = a;
+        }
+        v[j] = a;
+        ss = fmaf(a, a, ss);
+    }
+    if (!w) return;
+    ss = vt_wave_sum(ss);
+    if (vt_lane() == 0) red[vt_wave()] = ss;
+    __syncthreads();
+    const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+    const float inv = 1.0f / sqrtf(tot / (float)VT_DIM + eps);
+#pragma unroll
+    for (int j = 0; j < VT_DIM / 256; j++) {
+        const int c = (int)threadIdx.x + 256 * j;
+        unsigned h, l;
+        vt_split_planes(__fmul_rn(__fmul_rn(v[j], inv), w[c]), h, l);
+        hi[row * VT_DIM + c] = (uint16_t)h;
+        lo[row * VT_DIM + c] = (uint16_t)l;
+    }
+}
+
+void vt_launch_residual_norm_split(float *d_x, const float *d_part, int splits, size_t part_stride,
+                                   const float *d_w, uint16_t *d_hi, uint16_t *d_lo, int rows) {
+    hipLaunchKernelGGL(vt_residual_norm_split_kernel, dim3(rows), dim3(256), 0, g_vt.stream, d_x, d_part,
+                       splits, part_stride, d_w, d_hi, d_lo, VT_EPS);
+}
+
+/* gu [rows, 2*ffn] with (gate, up) adjacent -> (hi, lo) planes of silu(gate)*up
+ * (voxtral_tts_llm.c:346-350 on the row-interleaved gate/up matrix). */
+__global__ void vt_swiglu_split_kernel(uint16_t *hi, uint16_t *lo, const float *gu, size_t n2) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n2;
+         i += (size_t)gridDim.x * blockDim.x) {
+        const f32x4 g = reinterpret_cast<const f32x4 *>(gu)[i];
+        const float a = __fmul_rn(__fdiv_rn(g.x, __fadd_rn(1.0f, expf(-g.x))), g.y);
+        const float b = __fmul_rn(__fdiv_rn(g.z, __fadd_rn(1.0f, expf(-g.z))), g.w);
+        unsigned h0, l0, h1, l1;
+        vt_split_planes(a, h0, l0);
+        vt_split_planes(b, h1, l1);
+        reinterpret_cast<unsigned *>(hi)[i] = h0 | (h1 << 16);
+        reinterpret_cast<unsigned *>(lo)[i] = l0 | (l1 << 16);
+    }
+}
+
+void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, size_t n_out) {
+    hipLaunchKernelGGL(vt_swiglu_split_kernel, dim3(gm_blocks(n_out / 2)), dim3(256), 0, g_vt.stream, d_hi, d_lo,
+                       d_gu, n_out / 2);
+}
+
+/* C = sum of `splits` partial planes (fixed order), for callers that want the plain product. */
+__global__ void vt_sum_planes_kernel(float *out, const float *part, int splits, size_t stride, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (size_t)gridDim.x * blockDim.x) {
+        float p = part[i];
+        for (int s = 1; s < splits; s++) p = __fadd_rn(p, part[(size_t)s * stride + i]);
+        out[i] = p;
+    }
+}
+
+void vt_launch_sum_planes(float *d_out, const float *d_part, int splits, size_t stride, size_t n) {
+    hipLaunchKernelGGL(vt_sum_planes_kernel, dim3(gm_blocks(n)), dim3(256), 0, g_vt.stream, d_out, d_part,
+                       splits, stride, n);
+}

@@ -13,33 +13,6 @@
 #include <math.h>
 #include <string.h>
 
-/* qkv [S,6144] -> q [S,4096] (RoPE), cache rows start_pos.. (k with RoPE, v) */
-__global__ void vt_split_qkv_rope_kernel(const float *qkv, float *q, float *kc, float *vc,
-                                         const float *rope, int start_pos, int S) {
-    const int pairs = VT_QKV_DIM / 2;
-    const size_t total = (size_t)S * pairs;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-         i += (size_t)gridDim.x * blockDim.x) {
-        const int s = (int)(i / pairs), g = (int)(i % pairs) * 2;
-        const float a = qkv[(size_t)s * VT_QKV_DIM + g], b = qkv[(size_t)s * VT_QKV_DIM + g + 1];
-        if (g < VT_Q_DIM + VT_KV_DIM) {
-            const float *cs = rope + (size_t)(start_pos + s) * VT_HEAD_DIM;
-            const int d = (g & (VT_HEAD_DIM - 1)) >> 1;
-            const float c = cs[2 * d], sn = cs[2 * d + 1];
-            const float o0 = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn));
-            const float o1 = __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c));
-            float *dst = g < VT_Q_DIM ? q + (size_t)s * VT_Q_DIM + g
-                                      : kc + (size_t)(start_pos + s) * VT_KV_DIM + (g - VT_Q_DIM);
-            dst[0] = o0;
-            dst[1] = o1;
-        } else {
-            float *dst = vc + (size_t)(start_pos + s) * VT_KV_DIM + (g - VT_Q_DIM - VT_KV_DIM);
-            dst[0] = a;
-            dst[1] = b;
-        }
-    }
-}
-
 /* gu [S,18432] with (gate, up) adjacent -> h [S,9216] = silu(gate)*up */
 __global__ void vt_swiglu_pairs_kernel(const float *gu, float *h, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
@@ -76,12 +49,7 @@ static void seq_layer(const vt_layer_dev *L, float *x, const vt_seq_bufs *b, int
     const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
     vt_launch_rms_norm(b->xn, x, L->attn_norm, S, VT_DIM, VT_EPS);
     vt_launch_linear(b->qkv, b->xn, L->wqkv, NULL, S, VT_DIM, VT_QKV_DIM);
-    if (kc) {
-        hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(blocks_for((size_t)S * VT_QKV_DIM / 2)), dim3(256),
-                           0, st, b->qkv, b->q, kc, vc, g_vt.d_rope, start_pos, S);
-        vt_launch_attention(b->att, b->q, kc, vc, S, start_pos, start_pos + S, 1, VT_HEADS, VT_KV_HEADS,
-                            VT_HEAD_DIM, scale, VT_KV_DIM, VT_Q_DIM);
-    } else {
+    {
         for (int g0 = 0; g0 < S; g0 += group)
             vt_launch_attention(b->att + (size_t)g0 * VT_Q_DIM, b->qkv + (size_t)g0 * VT_QKV_DIM,
                                 b->qkv + (size_t)g0 * VT_QKV_DIM + VT_Q_DIM,
@@ -96,36 +64,6 @@ static void seq_layer(const vt_layer_dev *L, float *x, const vt_seq_bufs *b, int
                        b->gu, b->h, (size_t)S * VT_FFN);
     vt_launch_linear(b->proj, b->h, L->w2, NULL, S, VT_FFN, VT_DIM);
     vt_launch_add(x, b->proj, S * VT_DIM);
-}
-
-/* ---- backbone prefill ------------------------------------------------------------ */
-
-extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int start_pos, float *out_x) {
-    if (!g_vt.initialized || g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_llm_prefill: no weights uploaded"); return; }
-    if (seq_len < 1 || start_pos < 0 || start_pos + seq_len > g_vt.kv_max) {
-        vt_set_error("tts_hip_llm_prefill: rows [%d, %d) outside the KV cache (max %d)", start_pos,
-                     start_pos + seq_len, g_vt.kv_max);
-        return;
-    }
-    const int S = seq_len;
-    float *base = (float *)vt_scratch(sizeof(float) * (seq_floats(S) + (size_t)S * VT_DIM));
-    if (!base) return;
-    float *x = base;
-    vt_seq_bufs b;
-    carve(&b, base + (size_t)S * VT_DIM, S);
-    VT_TRYV(hipMemcpyAsync(x, embeds, sizeof(float) * (size_t)S * VT_DIM, hipMemcpyDefault, g_vt.stream));
-    for (int l = 0; l < g_vt.n_dec_layers; l++) {
-        float *kc = g_hip.kv_cache_k_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
-        float *vc = g_hip.kv_cache_v_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
-        seq_layer(&g_vt.h_layers[l], x, &b, S, kc, vc, start_pos, 0);
-    }
-    VT_TRYV(hipGetLastError());
-    VT_TRYV(hipStreamSynchronize(g_vt.stream));
-    if (out_x) VT_TRYV(hipMemcpy(out_x, x, sizeof(float) * (size_t)S * VT_DIM, hipMemcpyDefault));
-}
-
-extern "C" void tts_hip_llm_prefill(const float *embeds, int seq_len, int start_pos) {
-    tts_hip_llm_prefill_out(embeds, seq_len, start_pos, NULL);
 }
 
 /* ---- acoustic transformer --------------------------------------------------------- */

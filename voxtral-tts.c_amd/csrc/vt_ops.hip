@@ -7,6 +7,7 @@
  * vt_decode.hip / vt_prefill.hip / vt_acoustic.hip.
  */
 #include "vt_state.h"
+#include "vt_gemm.h"
 
 #include <math.h>
 #include <stdlib.h>
@@ -68,6 +69,30 @@ void vt_launch_linear(float *d_y, const float *d_x, const uint16_t *d_W, const f
                            seq_len, in_dim, out_dim, vec_ok);
 }
 
+/* Rows of activations against an aligned weight matrix go to the matrix cores:
+ * (hi, lo) planes of x, K cut into enough ranges to fill the device, partial
+ * planes summed in a fixed order.  Returns 0 when the shape does not qualify. */
+static int linear_mfma(float *d_y, const float *d_x, const uint16_t *d_W, int seq_len, int in_dim, int out_dim) {
+    if (seq_len < 8 || !vt_gemm_shape_ok(seq_len, out_dim, in_dim, 1) ||
+        (((uintptr_t)d_W | (uintptr_t)d_x | (uintptr_t)d_y) & 15))
+        return 0;
+    const int tiles = ((seq_len + 127) / 128) * (out_dim / 128);
+    int splits = 1;
+    static const int cand[] = {2, 3, 4, 6, 8};
+    for (int i = 0; i < 5 && tiles * splits < 192; i++)
+        if (vt_gemm_shape_ok(seq_len, out_dim, in_dim, cand[i])) splits = cand[i];
+    const size_t n_in = (size_t)seq_len * in_dim, n_out = (size_t)seq_len * out_dim;
+    const size_t part_bytes = splits > 1 ? sizeof(float) * n_out * splits : 0;
+    unsigned char *base = (unsigned char *)vt_scratch(part_bytes + 2 * sizeof(uint16_t) * n_in);
+    if (!base) return -1;
+    float *part = splits > 1 ? (float *)base : d_y;
+    uint16_t *hi = (uint16_t *)(base + part_bytes), *lo = hi + n_in;
+    vt_launch_split(hi, lo, d_x, n_in);
+    vt_launch_gemm(part, hi, lo, d_W, seq_len, out_dim, in_dim, splits);
+    if (splits > 1) vt_launch_sum_planes(d_y, part, splits, n_out, n_out);
+    return 1;
+}
+
 static int is_device_ptr(const void *p) {
     hipPointerAttribute_t at;
     if (hipPointerGetAttributes(&at, p) != hipSuccess) {
@@ -101,7 +126,11 @@ extern "C" void tts_hip_linear_bf16(float *y, const float *x, const uint16_t *W_
         if (!(tmp_y = vt_dev_alloc(yb))) goto done;
         dy = (float *)tmp_y;
     }
-    vt_launch_linear(dy, dx, (const uint16_t *)dW, NULL, seq_len, in_dim, out_dim);
+    {
+        const int r = linear_mfma(dy, dx, (const uint16_t *)dW, seq_len, in_dim, out_dim);
+        if (r < 0) goto done;
+        if (r == 0) vt_launch_linear(dy, dx, (const uint16_t *)dW, NULL, seq_len, in_dim, out_dim);
+    }
     if (!y_dev || tmp_x || tmp_W) {
         if (vt_check(hipStreamSynchronize(g_vt.stream), "linear sync")) goto done;
         if (!y_dev) (void)vt_check(hipMemcpy(y, dy, yb, hipMemcpyDeviceToHost), "linear y download");
@@ -290,6 +319,11 @@ extern "C" void tts_hip_causal_attention_prefill(float *d_out, const float *d_Q,
     if (!attn_args_ok("tts_hip_causal_attention_prefill", seq_len, start_pos + seq_len, n_heads,
                       n_kv_heads, head_dim)) return;
     if (start_pos < 0) { vt_set_error("tts_hip_causal_attention_prefill: negative start_pos"); return; }
+    if (n_heads == VT_HEADS && n_kv_heads == VT_KV_HEADS && head_dim == VT_HEAD_DIM && seq_len >= 8 &&
+        !(((uintptr_t)d_out | (uintptr_t)d_Q | (uintptr_t)d_K | (uintptr_t)d_V) & 15)) {
+        vt_launch_prefill_attention(d_out, NULL, NULL, d_Q, VT_Q_DIM, d_K, d_V, seq_len, start_pos);
+        return;
+    }
     vt_launch_attention(d_out, d_Q, d_K, d_V, seq_len, start_pos, start_pos + seq_len, 1, n_heads,
                         n_kv_heads, head_dim, scale, n_kv_heads * head_dim, n_heads * head_dim);
 }

@@ -1,0 +1,308 @@
+/*
+ * vt_prefill.hip - backbone prefill over a row block of the sequence (replaces
+ * tts_cuda_llm_prefill, voxtral_tts_cuda.cu:806-893; the layer follows
+ * voxtral_tts_llm.c:299-366).
+ *
+ * Per layer: RMSNorm into (hi, lo) bf16 planes -> q|k|v product on the matrix
+ * cores -> RoPE + cache append -> causal attention on the fp32 matrix cores
+ * -> output projection (K split in 2) -> residual + RMSNorm -> gate/up product
+ * -> SiLU*up -> down projection (K split in 3) -> residual fused with the next
+ * layer's RMSNorm.  Weights are the fused layouts of the decode path.
+ */
+#include "vt_state.h"
+#include "vt_gemm.h"
+
+#include <math.h>
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+/* ---- RoPE + cache append ------------------------------------------------------- */
+
+/* qkv [S,6144] -> q [S,4096] with RoPE, cache rows start_pos.. (k with RoPE, v) */
+__global__ void vt_split_qkv_rope_kernel(const float *qkv, float *q, float *kc, float *vc,
+                                         const float *rope, int start_pos, int S) {
+    const int pairs = VT_QKV_DIM / 2;
+    const size_t total = (size_t)S * pairs;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (size_t)gridDim.x * blockDim.x) {
+        const int s = (int)(i / pairs), g = (int)(i % pairs) * 2;
+        const f32x2 ab = *reinterpret_cast<const f32x2 *>(qkv + (size_t)s * VT_QKV_DIM + g);
+        f32x2 o = ab;
+        float *dst;
+        if (g < VT_Q_DIM + VT_KV_DIM) {
+            const float *cs = rope + (size_t)(start_pos + s) * VT_HEAD_DIM;
+            const int d = (g & (VT_HEAD_DIM - 1)) >> 1;
+            const float c = cs[2 * d], sn = cs[2 * d + 1];
+            o.x = __fsub_rn(__fmul_rn(ab.x, c), __fmul_rn(ab.y, sn));
+            o.y = __fadd_rn(__fmul_rn(ab.x, sn), __fmul_rn(ab.y, c));
+            dst = g < VT_Q_DIM ? q + (size_t)s * VT_Q_DIM + g
+                               : kc + (size_t)(start_pos + s) * VT_KV_DIM + (g - VT_Q_DIM);
+        } else {
+            dst = vc + (size_t)(start_pos + s) * VT_KV_DIM + (g - VT_Q_DIM - VT_KV_DIM);
+        }
+        *reinterpret_cast<f32x2 *>(dst) = o;
+    }
+}
+
+/* ---- causal attention, 32 queries x 32 keys per matrix-core tile --------------
+ * (tts_causal_attention, voxtral_tts_kernels.c:403-465, for head_dim 128 and four
+ * query heads per KV head.)
+ *
+ * Workgroup = (KV head, block of 32 queries), 4*NSPLIT waves: wave = (query head
+ * of the group, key-tile residue).  The waves of one residue share 32-key K and V
+ * tiles in LDS.  Scores are computed transposed, S^T = K Q^T, with
+ * v_mfma_f32_32x32x2_f32, so that a lane owns one query: lane l holds query l%32
+ * and the keys 8*(v/4) + 4*(l/32) + v%4 of the tile in accumulator element v.
+ * The softmax state is then per lane (one exchange with lane l^32 per tile), and
+ * the probabilities are already in the operand layout of the second product
+ * O^T = V^T P^T, whose reduction index runs over the keys in that same order.
+ * fp32 operands throughout.  Residues are merged through LDS at the end. */
+#define PA_KP 132                 /* K tile pitch in floats: 16-byte reads over keys cover all banks */
+#define PA_VP 136                 /* V tile pitch: lanes l and l^32 (4 keys apart) use disjoint banks */
+#define PA_TILE_FLOATS (32 * PA_KP + 32 * PA_VP)
+
+template <int NSPLIT>
+__global__ void __launch_bounds__(256 * NSPLIT)
+vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, const float *Q,
+                            int q_stride, const float *Kc, const float *Vc, int S,
+                            int start_pos, float scale) {
+    extern __shared__ __attribute__((aligned(16))) float pa_lds[];
+    const int g = (int)blockIdx.x, qt = (int)blockIdx.y;
+    const int t = (int)threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int hq = wave & 3, pz = wave >> 2;
+    const int tl = (hq << 6) | lane;                     /* thread index inside the residue group */
+    const int hh = lane >> 5, qi = lane & 31;
+    const int q0 = qt * 32;
+    const int my_q = q0 + qi;
+    const int head = g * 4 + hq;
+    float *Kt = pa_lds + (size_t)pz * PA_TILE_FLOATS, *Vt = Kt + 32 * PA_KP;
+
+    /* this lane's query: dims 64*hh .. 64*hh+63 */
+    float qreg[64];
+    {
+        const float *qp = Q + (size_t)(my_q < S ? my_q : S - 1) * q_stride + head * VT_HEAD_DIM + 64 * hh;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const f32x4 v = reinterpret_cast<const f32x4 *>(qp)[i];
+            qreg[4 * i] = v.x; qreg[4 * i + 1] = v.y; qreg[4 * i + 2] = v.z; qreg[4 * i + 3] = v.w;
+        }
+    }
+    f32x16 o[4];
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) o[b][v] = 0.f;
+    float m = -1e30f, lsum = 0.f;
+
+    const int last_q = (q0 + 31 < S ? q0 + 31 : S - 1) + start_pos;
+    const int ntiles = last_q / 32 + 1;                  /* key tiles 0 .. ntiles-1 are visible */
+    const int nsteps = (ntiles + NSPLIT - 1) / NSPLIT;
+    const int kv_rows = start_pos + S;
+
+    /* staging: the 256 threads of a residue group move 32 rows x 512 B of K and of V */
+    f32x4 rk[4], rv[4];
+    auto fetch = [&](int tile) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int c = tl + 256 * i, row = c >> 5, col = (c & 31) * 4;
+            int kr = tile * 32 + row;
+            if (kr >= kv_rows) kr = kv_rows - 1;
+            rk[i] = *reinterpret_cast<const f32x4 *>(Kc + (size_t)kr * VT_KV_DIM + g * VT_HEAD_DIM + col);
+            rv[i] = *reinterpret_cast<const f32x4 *>(Vc + (size_t)kr * VT_KV_DIM + g * VT_HEAD_DIM + col);
+        }
+    };
+    if (pz < ntiles) fetch(pz);
+
+    for (int step = 0; step < nsteps; step++) {
+        const int tile = step * NSPLIT + pz;
+        const bool valid = tile < ntiles;
+        __syncthreads();
+        if (valid) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = tl + 256 * i, row = c >> 5, col = (c & 31) * 4;
+                *reinterpret_cast<f32x4 *>(Kt + row * PA_KP + col) = rk[i];
+                *reinterpret_cast<f32x4 *>(Vt + row * PA_VP + col) = rv[i];
+            }
+        }
+        __syncthreads();
+        if (tile + NSPLIT < ntiles) fetch(tile + NSPLIT);
+        if (!valid) continue;
+
+        /* S^T = K Q^T over d = 64*hh + ks */
+        f32x16 s;
+#pragma unroll
+        for (int v = 0; v < 16; v++) s[v] = 0.f;
+#pragma unroll
+        for (int gk = 0; gk < 16; gk++) {
+            const f32x4 kf = *reinterpret_cast<const f32x4 *>(Kt + qi * PA_KP + 64 * hh + 4 * gk);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qreg[4 * gk], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qreg[4 * gk + 1], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qreg[4 * gk + 2], s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qreg[4 * gk + 3], s, 0, 0, 0);
+        }
+        /* online softmax for this lane's query */
+        const int qpos = start_pos + my_q;
+        float mx = -1e30f;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const int kpos = tile * 32 + 8 * (v >> 2) + 4 * hh + (v & 3);
+            s[v] = kpos <= qpos ? __fmul_rn(s[v], scale) : -3e38f;
+            mx = fmaxf(mx, s[v]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float mn = fmaxf(m, mx);
+        const float corr = __expf(m - mn);
+        float psum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            s[v] = s[v] > -1e38f ? __expf(s[v] - mn) : 0.f;
+            psum += s[v];
+        }
+        lsum = fmaf(lsum, corr, psum);
+        m = mn;
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) o[b][v] *= corr;
+        /* O^T += V^T P^T: reduction step ks pairs key 8*(ks/4) + 4*hh + ks%4 with s[ks] */
+#pragma unroll
+        for (int ks = 0; ks < 16; ks++) {
+            const float *vrow = Vt + (8 * (ks >> 2) + 4 * hh + (ks & 3)) * PA_VP + qi;
+#pragma unroll
+            for (int b = 0; b < 4; b++)
+                o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * b], s[ks], o[b], 0, 0, 0);
+        }
+    }
+
+    /* merge the residues: residue r > 0 parks (m, l, O) in LDS, residue 0 folds them in */
+    if (NSPLIT > 1) {
+        __syncthreads();
+        float *park = pa_lds;                            /* [NSPLIT-1][4 heads][66][64 lanes] */
+        for (int r = 1; r < NSPLIT; r++) {
+            float *slot = park + ((size_t)((r - 1) * 4 + hq) * 66) * 64 + lane;
+            if (pz == r) {
+                slot[0] = m;
+                slot[64] = lsum;
+#pragma unroll
+                for (int b = 0; b < 4; b++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) slot[(2 + b * 16 + v) * 64] = o[b][v];
+            }
+            __syncthreads();
+            if (pz == 0) {
+                const float m2 = slot[0], l2 = slot[64];
+                const float mn = fmaxf(m, m2);
+                const float c1 = __expf(m - mn), c2 = __expf(m2 - mn);
+                lsum = fmaf(lsum, c1, l2 * c2);
+                m = mn;
+#pragma unroll
+                for (int b = 0; b < 4; b++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) o[b][v] = fmaf(o[b][v], c1, slot[(2 + b * 16 + v) * 64] * c2);
+            }
+            __syncthreads();
+        }
+    }
+    if (pz != 0 || my_q >= S) return;
+    const float L = lsum + __shfl_xor(lsum, 32);
+    const float inv = L > 0.f ? __fdiv_rn(1.0f, L) : 0.f;
+    const size_t ob = (size_t)my_q * VT_Q_DIM + head * VT_HEAD_DIM;
+#pragma unroll
+    for (int b = 0; b < 4; b++)
+#pragma unroll
+        for (int v4 = 0; v4 < 4; v4++) {
+            const int d = 32 * b + 8 * v4 + 4 * hh;
+            f32x4 r;
+            r.x = __fmul_rn(o[b][4 * v4], inv);
+            r.y = __fmul_rn(o[b][4 * v4 + 1], inv);
+            r.z = __fmul_rn(o[b][4 * v4 + 2], inv);
+            r.w = __fmul_rn(o[b][4 * v4 + 3], inv);
+            if (out) *reinterpret_cast<f32x4 *>(out + ob + d) = r;
+            if (out_hi) {
+                unsigned h0, l0, h1, l1, h2, l2, h3, l3;
+                vt_split_planes(r.x, h0, l0);
+                vt_split_planes(r.y, h1, l1);
+                vt_split_planes(r.z, h2, l2);
+                vt_split_planes(r.w, h3, l3);
+                u32x2 ph = {h0 | (h1 << 16), h2 | (h3 << 16)}, pl = {l0 | (l1 << 16), l2 | (l3 << 16)};
+                *reinterpret_cast<u32x2 *>(out_hi + ob + d) = ph;
+                *reinterpret_cast<u32x2 *>(out_lo + ob + d) = pl;
+            }
+        }
+}
+
+#define PA_NSPLIT 2
+
+static size_t pa_lds_bytes(int nsplit) {
+    size_t tiles = sizeof(float) * (size_t)nsplit * PA_TILE_FLOATS;
+    size_t park = sizeof(float) * (size_t)(nsplit - 1) * 4 * 66 * 64;
+    return tiles > park ? tiles : park;
+}
+
+/* Q rows are q_stride floats apart; out / (out_hi, out_lo) are [S,4096], each optional. */
+void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
+                                 int q_stride, const float *d_K, const float *d_V, int S, int start_pos) {
+    const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
+    static int attr_set = 0;
+    if (!attr_set) {
+        if (vt_check(hipFuncSetAttribute((const void *)vt_prefill_attention_kernel<PA_NSPLIT>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)pa_lds_bytes(PA_NSPLIT)), "attention LDS size"))
+            return;
+        attr_set = 1;
+    }
+    hipLaunchKernelGGL(vt_prefill_attention_kernel<PA_NSPLIT>, dim3(VT_KV_HEADS, (S + 31) / 32),
+                       dim3(256 * PA_NSPLIT), pa_lds_bytes(PA_NSPLIT), g_vt.stream, d_out, d_hi, d_lo, d_Q,
+                       q_stride, d_K, d_V, S, start_pos, scale);
+}
+
+/* ---- backbone prefill ------------------------------------------------------------ */
+
+static int ew_blocks(size_t n) { size_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : b); }
+
+extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int start_pos, float *out_x) {
+    if (!g_vt.initialized || g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_llm_prefill: no weights uploaded"); return; }
+    if (seq_len < 1 || start_pos < 0 || start_pos + seq_len > g_vt.kv_max) {
+        vt_set_error("tts_hip_llm_prefill: rows [%d, %d) outside the KV cache (max %d)", start_pos,
+                     start_pos + seq_len, g_vt.kv_max);
+        return;
+    }
+    const size_t S = (size_t)seq_len;
+    hipStream_t st = g_vt.stream;
+    /* work area: x | wide f32 (qkv or gate/up) | q | partial planes | hi | lo */
+    const size_t n_x = S * VT_DIM, n_wide = S * 2 * VT_FFN, n_q = S * VT_Q_DIM, n_part = 3 * S * VT_DIM;
+    const size_t n_plane = S * VT_FFN;                            /* bf16 elements per plane */
+    const size_t bytes = sizeof(float) * (n_x + n_wide + n_q + n_part) + 2 * sizeof(uint16_t) * n_plane;
+    float *x = (float *)vt_scratch(bytes);
+    if (!x) return;
+    float *wide = x + n_x, *q = wide + n_wide, *part = q + n_q;
+    uint16_t *hi = (uint16_t *)(part + n_part), *lo = hi + n_plane;
+    const size_t ps = S * VT_DIM;
+
+    VT_TRYV(hipMemcpyAsync(x, embeds, sizeof(float) * n_x, hipMemcpyDefault, st));
+    vt_launch_residual_norm_split(x, NULL, 0, 0, g_vt.h_layers[0].attn_norm, hi, lo, seq_len);
+    for (int l = 0; l < g_vt.n_dec_layers; l++) {
+        const vt_layer_dev *L = &g_vt.h_layers[l];
+        float *kc = g_hip.kv_cache_k_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
+        float *vc = g_hip.kv_cache_v_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
+        vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, 1);
+        hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(ew_blocks(S * VT_QKV_DIM / 2)), dim3(256), 0, st,
+                           wide, q, kc, vc, g_vt.d_rope, start_pos, seq_len);
+        vt_launch_prefill_attention(NULL, hi, lo, q, VT_Q_DIM, kc, vc, seq_len, start_pos);
+        vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, 2);
+        vt_launch_residual_norm_split(x, part, 2, ps, L->ffn_norm, hi, lo, seq_len);
+        vt_launch_gemm(wide, hi, lo, L->w13, seq_len, 2 * VT_FFN, VT_DIM, 1);
+        vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN);
+        vt_launch_gemm(part, hi, lo, L->w2, seq_len, VT_DIM, VT_FFN, 3);
+        const float *next_norm = l + 1 < g_vt.n_dec_layers ? g_vt.h_layers[l + 1].attn_norm : NULL;
+        vt_launch_residual_norm_split(x, part, 3, ps, next_norm, hi, lo, seq_len);
+    }
+    VT_TRYV(hipGetLastError());
+    VT_TRYV(hipStreamSynchronize(st));
+    if (out_x) VT_TRYV(hipMemcpy(out_x, x, sizeof(float) * n_x, hipMemcpyDefault));
+}
+
+extern "C" void tts_hip_llm_prefill(const float *embeds, int seq_len, int start_pos) {
+    tts_hip_llm_prefill_out(embeds, seq_len, start_pos, NULL);
+}

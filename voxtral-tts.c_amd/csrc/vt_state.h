@@ -89,6 +89,8 @@ void vt_launch_attention(float *d_out, const float *d_Q, const float *d_K, const
                          int seq_q, int q_offset, int seq_k, int causal, int n_heads,
                          int n_kv_heads, int head_dim, float scale, int kv_stride, int q_stride);
 void vt_launch_add(float *d_a, const float *d_b, int n);
+void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
+                                 int q_stride, const float *d_K, const float *d_V, int S, int start_pos);
 int vt_stream_supported(void);
 int vt_run_step_stream(const vt_step_args &a);
 int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
