@@ -158,7 +158,7 @@ extern "C" void tts_hip_free(void) {
     void *ptrs[] = {g_vt.d_layers, g_vt.d_dec_norm, g_vt.d_tok_emb, g_vt.ac.input_proj,
                     g_vt.ac.time_proj, g_vt.ac.llm_proj, g_vt.ac.semantic_out,
                     g_vt.ac.acoustic_out, g_vt.ac.semantic_bias, g_vt.ac.norm,
-                    g_vt.ac.time_inv_freq, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu,
+                    g_vt.ac.time_inv_freq, g_vt.ac.time_tok, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu,
                     g_vt.d_rope, g_vt.d_x, g_vt.d_q, g_vt.d_attn, g_vt.d_h, g_vt.d_att_part,
                     g_vt.d_att_cnt, g_vt.d_embed, g_vt.d_hidden, g_vt.d_bar_flags,
                     g_vt.d_abort, g_vt.d_dummy, g_vt.d_scratch};
@@ -278,10 +278,12 @@ extern "C" int tts_hip_upload_acoustic_weights(void *acoustic_ptr) {
     if (!ac) { vt_set_error("tts_hip_upload_acoustic_weights: NULL"); return -1; }
     vt_acoustic_dev *d = &g_vt.ac;
     void *old[] = {d->input_proj, d->time_proj, d->llm_proj, d->semantic_out, d->acoustic_out,
-                   d->semantic_bias, d->norm, d->time_inv_freq};
+                   d->semantic_bias, d->norm, d->time_inv_freq, d->time_tok};
     for (size_t i = 0; i < sizeof old / sizeof old[0]; i++) if (old[i]) (void)hipFree(old[i]);
     g_vt.ac_uploaded = 0;
     d->semantic_bias = NULL;
+    d->time_tok_ready = 0;
+    if (!(d->time_tok = (float *)vt_dev_alloc(sizeof(float) * 7 * VT_DIM))) return -1;
     if (!(d->input_proj = (uint16_t *)upload(ac->input_proj_bf16, (size_t)VT_DIM * VT_AC_DIM_IN * 2))) return -1;
     if (!(d->time_proj = (uint16_t *)upload(ac->time_proj_bf16, (size_t)VT_DIM * VT_DIM * 2))) return -1;
     if (!(d->llm_proj = (uint16_t *)upload(ac->llm_proj_bf16, (size_t)VT_DIM * VT_DIM * 2))) return -1;

@@ -4,7 +4,7 @@
  * bf16-weight linear, RMSNorm, RoPE, SiLU*mul, residual add, attention
  * (decode / causal prefill / bidirectional) and embedding lookup.
  * Shapes are arbitrary here; the fixed-shape fused paths live in
- * vt_decode.hip / vt_prefill.hip / vt_acoustic.hip.
+ * vt_decode.hip, vt_prefill.hip and vt_acoustic.hip.
  */
 #include "vt_state.h"
 #include "vt_gemm.h"

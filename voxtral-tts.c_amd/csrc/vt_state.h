@@ -27,6 +27,8 @@ struct vt_acoustic_dev {
     float *norm;
     float *time_inv_freq;
     float h_time_inv_freq[VT_DIM / 2];
+    float *time_tok;              /* [7, 3072] projected time tokens of the Euler grid */
+    int time_tok_ready;
 };
 
 struct vt_state {
