@@ -12,8 +12,8 @@
  *
  * A layer is four kernels, each a skinny product on the matrix cores
  * (v_mfma_f32_16x16x32_bf16, the 6 activation rows as (hi, lo) bf16 planes in
- * LDS, 16 weight rows per workgroup streamed straight from HBM into the B
- * operand, the 8 waves of a workgroup splitting K):
+ * LDS, 12 weight rows at a time streamed straight from HBM into the B operand
+ * by one persistent workgroup per CU, its 8 waves splitting K):
  *   RMSNorm + q|k|v            -> qkv [6, 6144]
  *   attention (3x3 per head and branch) + output projection + residual
  *   RMSNorm + gate/up + SiLU*up -> h [6, 9216]
@@ -28,6 +28,12 @@
 #include <string.h>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(1))) const u32x4 ac_gptr_u32x4;
+
+/* Two consecutive 16-byte loads of a lane share a 128-byte line (a load instruction
+ * covers 16 weight rows x 64 bytes), so these are ordinary cached loads: the second
+ * one must find the line the first one brought in. */
+__device__ __forceinline__ u32x4 ac_ldw(const uint16_t *p) { return *(ac_gptr_u32x4 *)p; }
 
 #define AC_ROWS    6
 #define AC_THREADS 512
@@ -51,29 +57,43 @@ template <int PH> struct ac_shape {
     static constexpr int NL = KW / 32;                               /* 16-byte loads per lane and pass */
     static constexpr int PITCH = KP * 2 + 16;                        /* bytes per plane row */
     static constexpr int PLANE = AC_ROWS * PITCH;
-    static constexpr int LDS_BYTES = 2 * PLANE + 4 * (AC_WAVES * AC_ROWS * 16 + AC_WAVES * 8);
+    static constexpr int LDS_BYTES = 2 * PLANE + 4 * (2 * AC_WAVES * AC_ROWS * 16 + AC_WAVES * 8);
 };
 
-/* rows of 3072 -> planes, optionally through RMSNorm.  Thread t owns the column
- * pairs 2t + 1024 j. */
-template <bool NORM>
-__device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned char *lo, int pitch,
-                                                  const float *src, int src_stride, const float *gain,
-                                                  float *red) {
+/* Activation rows are fetched into registers BEFORE the weight loads of a pass are
+ * issued: a wave's loads return in order, so this way the planes can be built while
+ * the weights are still streaming in. */
+struct ac_rows_regs { f32x2 v[AC_ROWS][3]; f32x2 g[3]; };
+struct ac_attn_regs { f32x4 q[3][4], k[3][4], v[3][4]; };
+
+/* rows of 3072: thread t owns the column pairs 2t + 1024 j */
+__device__ __forceinline__ void ac_fetch_rows(ac_rows_regs &r, const float *src, int src_stride,
+                                              const float *gain) {
     const int t = (int)threadIdx.x;
-    f32x2 v[AC_ROWS][3];
 #pragma unroll
     for (int m = 0; m < AC_ROWS; m++)
 #pragma unroll
         for (int j = 0; j < 3; j++)
-            v[m][j] = *reinterpret_cast<const f32x2 *>(src + (size_t)m * src_stride + 2 * t + 1024 * j);
+            r.v[m][j] = *reinterpret_cast<const f32x2 *>(src + (size_t)m * src_stride + 2 * t + 1024 * j);
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        r.g[j] = f32x2{1.f, 1.f};
+        if (gain) r.g[j] = *reinterpret_cast<const f32x2 *>(gain + 2 * t + 1024 * j);
+    }
+}
+
+/* registers -> (hi, lo) planes, optionally through RMSNorm */
+template <bool NORM>
+__device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned char *lo, int pitch,
+                                                  const ac_rows_regs &r, float *red) {
+    const int t = (int)threadIdx.x;
     float inv[AC_ROWS];
     if (NORM) {
 #pragma unroll
         for (int m = 0; m < AC_ROWS; m++) {
             float ss = 0.f;
 #pragma unroll
-            for (int j = 0; j < 3; j++) ss = fmaf(v[m][j].x, v[m][j].x, fmaf(v[m][j].y, v[m][j].y, ss));
+            for (int j = 0; j < 3; j++) ss = fmaf(r.v[m][j].x, r.v[m][j].x, fmaf(r.v[m][j].y, r.v[m][j].y, ss));
             ss = vt_wave_sum(ss);
             if (vt_lane() == 0) red[vt_wave() * 8 + m] = ss;
         }
@@ -89,11 +109,10 @@ __device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned ch
 #pragma unroll
     for (int j = 0; j < 3; j++) {
         const int c = 2 * t + 1024 * j;
-        f32x2 g = {1.f, 1.f};
-        if (NORM) g = *reinterpret_cast<const f32x2 *>(gain + c);
+        const f32x2 g = r.g[j];
 #pragma unroll
         for (int m = 0; m < AC_ROWS; m++) {
-            float a = v[m][j].x, b = v[m][j].y;
+            float a = r.v[m][j].x, b = r.v[m][j].y;
             if (NORM) {
                 a = __fmul_rn(__fmul_rn(a, inv[m]), g.x);
                 b = __fmul_rn(__fmul_rn(b, inv[m]), g.y);
@@ -110,25 +129,26 @@ __device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned ch
 /* Bidirectional attention over the 3 tokens of each branch, straight into the
  * planes that feed the output projection (tts_bidirectional_attention,
  * voxtral_tts_kernels.c:467-525).  8 lanes per (branch, head), 16 dims each. */
-__device__ __forceinline__ void ac_attention_to_planes(unsigned char *hi, unsigned char *lo, int pitch,
-                                                       const float *qkv) {
+__device__ __forceinline__ void ac_fetch_attn(ac_attn_regs &r, const float *qkv) {
     const int lane = vt_lane(), pair = vt_wave() * 8 + (lane >> 3), sub = lane & 7;
     const int br = pair >> 5, h = pair & 31, d0 = sub * 16;
-    const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
-    float q[3][16], k[3][16], v[3][16];
 #pragma unroll
     for (int i = 0; i < 3; i++) {
         const float *row = qkv + (size_t)(br * 3 + i) * VT_QKV_DIM;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const f32x4 a = *reinterpret_cast<const f32x4 *>(row + h * VT_HEAD_DIM + d0 + 4 * e);
-            const f32x4 b = *reinterpret_cast<const f32x4 *>(row + VT_Q_DIM + (h >> 2) * VT_HEAD_DIM + d0 + 4 * e);
-            const f32x4 c = *reinterpret_cast<const f32x4 *>(row + VT_Q_DIM + VT_KV_DIM + (h >> 2) * VT_HEAD_DIM + d0 + 4 * e);
-            q[i][4 * e] = a.x; q[i][4 * e + 1] = a.y; q[i][4 * e + 2] = a.z; q[i][4 * e + 3] = a.w;
-            k[i][4 * e] = b.x; k[i][4 * e + 1] = b.y; k[i][4 * e + 2] = b.z; k[i][4 * e + 3] = b.w;
-            v[i][4 * e] = c.x; v[i][4 * e + 1] = c.y; v[i][4 * e + 2] = c.z; v[i][4 * e + 3] = c.w;
+            r.q[i][e] = *reinterpret_cast<const f32x4 *>(row + h * VT_HEAD_DIM + d0 + 4 * e);
+            r.k[i][e] = *reinterpret_cast<const f32x4 *>(row + VT_Q_DIM + (h >> 2) * VT_HEAD_DIM + d0 + 4 * e);
+            r.v[i][e] = *reinterpret_cast<const f32x4 *>(row + VT_Q_DIM + VT_KV_DIM + (h >> 2) * VT_HEAD_DIM + d0 + 4 * e);
         }
     }
+}
+
+__device__ __forceinline__ void ac_attention_to_planes(unsigned char *hi, unsigned char *lo, int pitch,
+                                                       const ac_attn_regs &r) {
+    const int lane = vt_lane(), pair = vt_wave() * 8 + (lane >> 3), sub = lane & 7;
+    const int br = pair >> 5, h = pair & 31, d0 = sub * 16;
+    const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
 #pragma unroll
     for (int i = 0; i < 3; i++) {
         float s[3];
@@ -136,10 +156,15 @@ __device__ __forceinline__ void ac_attention_to_planes(unsigned char *hi, unsign
         for (int j = 0; j < 3; j++) {
             float p = 0.f;
 #pragma unroll
-            for (int e = 0; e < 16; e++) p = fmaf(q[i][e], k[j][e], p);
+            for (int e = 0; e < 4; e++) {
+                p = fmaf(r.q[i][e].x, r.k[j][e].x, p);
+                p = fmaf(r.q[i][e].y, r.k[j][e].y, p);
+                p = fmaf(r.q[i][e].z, r.k[j][e].z, p);
+                p = fmaf(r.q[i][e].w, r.k[j][e].w, p);
+            }
             p += vt_dpp<0xB1>(p);                 /* lanes ^1 */
             p += vt_dpp<0x4E>(p);                 /* lanes ^2 */
-            p += vt_dpp<0x141>(p);                /* the other half of the 8-lane group (row_half_mirror) */
+            p += vt_dpp<0x141>(p);                /* the other quad of the 8-lane group (row_half_mirror) */
             s[j] = __fmul_rn(p, scale);
         }
         const float mx = fmaxf(s[0], fmaxf(s[1], s[2]));
@@ -148,61 +173,56 @@ __device__ __forceinline__ void ac_attention_to_planes(unsigned char *hi, unsign
         unsigned char *ph = hi + (br * 3 + i) * pitch + 2 * (h * VT_HEAD_DIM + d0);
         unsigned char *pl = lo + (br * 3 + i) * pitch + 2 * (h * VT_HEAD_DIM + d0);
 #pragma unroll
-        for (int e = 0; e < 16; e += 2) {
-            const float o0 = __fmul_rn(fmaf(p2, v[2][e], fmaf(p1, v[1][e], p0 * v[0][e])), inv);
-            const float o1 = __fmul_rn(fmaf(p2, v[2][e + 1], fmaf(p1, v[1][e + 1], p0 * v[0][e + 1])), inv);
-            unsigned h0, l0, h1, l1;
+        for (int e = 0; e < 4; e++) {
+            const float o0 = __fmul_rn(fmaf(p2, r.v[2][e].x, fmaf(p1, r.v[1][e].x, p0 * r.v[0][e].x)), inv);
+            const float o1 = __fmul_rn(fmaf(p2, r.v[2][e].y, fmaf(p1, r.v[1][e].y, p0 * r.v[0][e].y)), inv);
+            const float o2 = __fmul_rn(fmaf(p2, r.v[2][e].z, fmaf(p1, r.v[1][e].z, p0 * r.v[0][e].z)), inv);
+            const float o3 = __fmul_rn(fmaf(p2, r.v[2][e].w, fmaf(p1, r.v[1][e].w, p0 * r.v[0][e].w)), inv);
+            unsigned h0, l0, h1, l1, h2, l2, h3, l3;
             vt_split_planes(o0, h0, l0);
             vt_split_planes(o1, h1, l1);
-            *reinterpret_cast<unsigned *>(ph + 2 * e) = h0 | (h1 << 16);
-            *reinterpret_cast<unsigned *>(pl + 2 * e) = l0 | (l1 << 16);
+            vt_split_planes(o2, h2, l2);
+            vt_split_planes(o3, h3, l3);
+            const u32x2 vh = {h0 | (h1 << 16), h2 | (h3 << 16)}, vl = {l0 | (l1 << 16), l2 | (l3 << 16)};
+            *reinterpret_cast<u32x2 *>(ph + 8 * e) = vh;
+            *reinterpret_cast<u32x2 *>(pl + 8 * e) = vl;
         }
     }
 }
 
-template <int PH>
-__global__ void __launch_bounds__(AC_THREADS)
-vt_ac_phase_kernel(ac_phase_args a) {
-    typedef ac_shape<PH> SH;
-    extern __shared__ __attribute__((aligned(16))) unsigned char ac_lds[];
-    unsigned char *hi = ac_lds, *lo = ac_lds + SH::PLANE;
-    float *red = reinterpret_cast<float *>(ac_lds + 2 * SH::PLANE);          /* [8 waves][6][16] */
-    float *red_ss = red + AC_WAVES * AC_ROWS * 16;                           /* [8 waves][8] */
-    const int lane = vt_lane(), wave = vt_wave();
-    const int col = lane & 15, kg = lane >> 4;
-    const int n0 = (int)blockIdx.x * 16;
-    const uint16_t *wrow = a.W + (size_t)(n0 + col) * SH::KTOT + wave * SH::KW + 8 * kg;
+/* One persistent workgroup per CU.  A unit is AC_RB consecutive weight rows (12 of the
+ * 16 columns of the matrix-core tile: 3072, 6144 and 18432 rows then split evenly over
+ * 256 CUs); units are dealt round-robin.  The activation planes are built once per
+ * workgroup, while the first unit's weights are already on their way; after that the
+ * weights of unit u+1 stream into one register set while unit u is multiplied out of
+ * the other.  The down projection (K = 9216) takes its K in three passes and rebuilds
+ * the planes for each. */
+#define AC_RB 12
 
-    u32x4 wreg[2][SH::NL];
+template <int PH, int NL>
+__device__ __forceinline__ void ac_issue(u32x4 (&wreg)[NL], const uint16_t *p) {
 #pragma unroll
-    for (int i = 0; i < SH::NL; i++) wreg[0][i] = vt_ldw(wrow + 32 * i);
+    for (int i = 0; i < NL; i++) wreg[i] = ac_ldw(p + 32 * i);
+}
 
-    f32x4 acc_hi = {0.f, 0.f, 0.f, 0.f}, acc_lo = {0.f, 0.f, 0.f, 0.f};
-    const int arow = col < AC_ROWS ? col : 0;          /* rows 6..15 of the A operand are don't-care */
-    const unsigned char *fa = hi + arow * SH::PITCH + 2 * (wave * SH::KW + 8 * kg);
-    const unsigned char *fl = lo + arow * SH::PITCH + 2 * (wave * SH::KW + 8 * kg);
-
+template <int NL>
+__device__ __forceinline__ void ac_consume(const u32x4 (&wreg)[NL], const unsigned char *fa, const unsigned char *fl,
+                                           f32x4 &acc_hi, f32x4 &acc_lo) {
 #pragma unroll
-    for (int pass = 0; pass < SH::NPASS; pass++) {
-        if (pass > 0) __syncthreads();                 /* every wave is done with the previous planes */
-        if (PH == AC_QKV || PH == AC_W13) ac_rows_to_planes<true>(hi, lo, SH::PITCH, a.in, VT_DIM, a.gain, red_ss);
-        if (PH == AC_W2) ac_rows_to_planes<false>(hi, lo, SH::PITCH, a.in + pass * SH::KP, VT_FFN, NULL, red_ss);
-        if (PH == AC_WO) ac_attention_to_planes(hi, lo, SH::PITCH, a.in);
-        __syncthreads();
-        if (pass + 1 < SH::NPASS) {
-#pragma unroll
-            for (int i = 0; i < SH::NL; i++) wreg[(pass + 1) & 1][i] = vt_ldw(wrow + (pass + 1) * SH::KP + 32 * i);
-        }
-#pragma unroll
-        for (int i = 0; i < SH::NL; i++) {
-            const bf16x8 b = __builtin_bit_cast(bf16x8, wreg[pass & 1][i]);
-            const bf16x8 xh = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(fa + 64 * i));
-            const bf16x8 xl = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(fl + 64 * i));
-            acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xl, b, acc_lo, 0, 0, 0);
-            acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xh, b, acc_hi, 0, 0, 0);
-        }
+    for (int i = 0; i < NL; i++) {
+        const bf16x8 b = __builtin_bit_cast(bf16x8, wreg[i]);
+        const bf16x8 xh = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(fa + 64 * i));
+        const bf16x8 xl = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4 *>(fl + 64 * i));
+        acc_lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xl, b, acc_lo, 0, 0, 0);
+        acc_hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xh, b, acc_hi, 0, 0, 0);
     }
+}
 
+/* cross-wave sum of one unit and its epilogue; `red` is this unit's buffer */
+template <int PH>
+__device__ __forceinline__ void ac_finish_unit(const ac_phase_args &a, float *red, int n0, f32x4 acc_hi,
+                                               f32x4 acc_lo) {
+    const int lane = vt_lane(), wave = vt_wave(), col = lane & 15, kg = lane >> 4;
     /* accumulator element v of lane l: activation row 4*(l/16) + v, weight row l%16 */
 #pragma unroll
     for (int v = 0; v < 4; v++) {
@@ -212,7 +232,7 @@ vt_ac_phase_kernel(ac_phase_args a) {
     __syncthreads();
     const int t = (int)threadIdx.x;
     if (PH == AC_W13) {
-        if (t < AC_ROWS * 8) {
+        if (t < AC_ROWS * 8 && (t & 7) < AC_RB / 2) {
             const int m = t >> 3, j = t & 7;
             float g = 0.f, u = 0.f;
 #pragma unroll
@@ -222,7 +242,7 @@ vt_ac_phase_kernel(ac_phase_args a) {
             }
             a.out[(size_t)m * VT_FFN + (n0 >> 1) + j] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
         }
-    } else if (t < AC_ROWS * 16) {
+    } else if (t < AC_ROWS * 16 && (t & 15) < AC_RB) {
         const int m = t >> 4, n = t & 15;
         float y = 0.f;
 #pragma unroll
@@ -232,6 +252,82 @@ vt_ac_phase_kernel(ac_phase_args a) {
         } else {
             float *p = a.out + (size_t)m * VT_DIM + n0 + n;
             *p = __fadd_rn(*p, y);
+        }
+    }
+}
+
+template <int PH>
+__global__ void __launch_bounds__(AC_THREADS)
+vt_ac_phase_kernel(ac_phase_args a, int n_units) {
+    typedef ac_shape<PH> SH;
+    extern __shared__ __attribute__((aligned(16))) unsigned char ac_lds[];
+    unsigned char *hi = ac_lds, *lo = ac_lds + SH::PLANE;
+    float *red = reinterpret_cast<float *>(ac_lds + 2 * SH::PLANE);          /* 2 x [8 waves][6][16] */
+    float *red_ss = red + 2 * AC_WAVES * AC_ROWS * 16;                       /* [8 waves][8] */
+    const int lane = vt_lane(), wave = vt_wave();
+    const int col = lane & 15, kg = lane >> 4;
+    const bool live = col < AC_RB;
+    const int G = (int)gridDim.x;
+    int u = (int)blockIdx.x;
+    if (u >= n_units) return;
+    /* this lane's weight row inside unit 0, at this wave's K slice; the four spare columns of
+     * the tile repeat row 0 (same cache lines, results unused) */
+    const uint16_t *wbase = a.W + (size_t)(live ? col : 0) * SH::KTOT + wave * SH::KW + 8 * kg;
+    const size_t unit_stride = (size_t)AC_RB * SH::KTOT;
+    const int arow = col < AC_ROWS ? col : 0;          /* rows 6..15 of the A operand are don't-care */
+    const unsigned char *fa = hi + arow * SH::PITCH + 2 * (wave * SH::KW + 8 * kg);
+    const unsigned char *fl = lo + arow * SH::PITCH + 2 * (wave * SH::KW + 8 * kg);
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    u32x4 w0[SH::NL], w1[SH::NL];
+
+    if (SH::NPASS == 1) {
+        ac_rows_regs rr;
+        ac_attn_regs ra;
+        if (PH == AC_WO) ac_fetch_attn(ra, a.in); else ac_fetch_rows(rr, a.in, VT_DIM, a.gain);
+        ac_issue<PH>(w0, wbase + u * unit_stride);
+        if (PH == AC_WO) ac_attention_to_planes(hi, lo, SH::PITCH, ra);
+        else ac_rows_to_planes<true>(hi, lo, SH::PITCH, rr, red_ss);
+        __syncthreads();
+        for (;;) {
+            {
+                const int nx = u + G;
+                if (nx < n_units) ac_issue<PH>(w1, wbase + nx * unit_stride);
+                f32x4 ah = zero4, al = zero4;
+                ac_consume(w0, fa, fl, ah, al);
+                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al);
+                u = nx;
+                if (u >= n_units) break;
+            }
+            {
+                const int nx = u + G;
+                if (nx < n_units) ac_issue<PH>(w0, wbase + nx * unit_stride);
+                f32x4 ah = zero4, al = zero4;
+                ac_consume(w1, fa, fl, ah, al);
+                ac_finish_unit<PH>(a, red + AC_WAVES * AC_ROWS * 16, u * AC_RB, ah, al);
+                u = nx;
+                if (u >= n_units) break;
+            }
+        }
+    } else {
+        for (; u < n_units; u += G) {
+            const uint16_t *wp = wbase + u * unit_stride;
+            ac_rows_regs rr;
+            ac_fetch_rows(rr, a.in, VT_FFN, NULL);
+            u32x4 wreg[2][SH::NL];
+            ac_issue<PH>(wreg[0], wp);
+            f32x4 ah = zero4, al = zero4;
+#pragma unroll
+            for (int pass = 0; pass < SH::NPASS; pass++) {
+                __syncthreads();                        /* nobody still reads the planes or red */
+                ac_rows_to_planes<false>(hi, lo, SH::PITCH, rr, red_ss);
+                __syncthreads();
+                if (pass + 1 < SH::NPASS) {
+                    ac_fetch_rows(rr, a.in + (pass + 1) * SH::KP, VT_FFN, NULL);
+                    ac_issue<PH>(wreg[(pass + 1) & 1], wp + (pass + 1) * SH::KP);
+                }
+                ac_consume(wreg[pass & 1], fa, fl, ah, al);
+            }
+            ac_finish_unit<PH>(a, red, u * AC_RB, ah, al);
         }
     }
 }
@@ -259,20 +355,23 @@ vt_ac_edge_kernel(ac_edge_args a) {
     __shared__ float s_inv[2];
     __shared__ float s_vel[2 * VT_AC_DIM_IN];
     __shared__ float s_x[VT_AC_DIM_IN];
+    __shared__ __attribute__((aligned(16))) float s_xn[2][VT_DIM];
     const int t = (int)threadIdx.x, lane = vt_lane(), wave = vt_wave();
     if (t < VT_AC_DIM_IN) s_x[t] = a.x[t];
     if (a.do_back) {
         /* final RMSNorm of token 0 of each branch (rows 0 and 3), then the 36-wide projection
          * (voxtral_tts_acoustic.c:255-261) */
-        float ss[2] = {0.f, 0.f};
+        float v[2][3];
 #pragma unroll
         for (int b = 0; b < 2; b++) {
-            for (int c = t; c < VT_DIM; c += 1024) {
-                const float v = a.tok_in[(size_t)(3 * b) * VT_DIM + c];
-                ss[b] = fmaf(v, v, ss[b]);
+            float ss = 0.f;
+#pragma unroll
+            for (int j = 0; j < 3; j++) {
+                v[b][j] = a.tok_in[(size_t)(3 * b) * VT_DIM + t + 1024 * j];
+                ss = fmaf(v[b][j], v[b][j], ss);
             }
-            ss[b] = vt_wave_sum(ss[b]);
-            if (lane == 0) red[b][wave] = ss[b];
+            ss = vt_wave_sum(ss);
+            if (lane == 0) red[b][wave] = ss;
         }
         __syncthreads();
         if (t < 2) {
@@ -281,13 +380,23 @@ vt_ac_edge_kernel(ac_edge_args a) {
             s_inv[t] = 1.0f / sqrtf(tot / (float)VT_DIM + VT_EPS);
         }
         __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            const float g = a.norm[t + 1024 * j];
+            s_xn[0][t + 1024 * j] = __fmul_rn(__fmul_rn(v[0][j], s_inv[0]), g);
+            s_xn[1][t + 1024 * j] = __fmul_rn(__fmul_rn(v[1][j], s_inv[1]), g);
+        }
+        __syncthreads();
         for (int o = wave; o < 2 * VT_AC_DIM_IN; o += 16) {
             const int b = o / VT_AC_DIM_IN, r = o % VT_AC_DIM_IN;
-            const float inv = s_inv[b];
             float acc = 0.f;
-            for (int c = lane; c < VT_DIM; c += 64) {
-                const float xn = __fmul_rn(__fmul_rn(a.tok_in[(size_t)(3 * b) * VT_DIM + c], inv), a.norm[c]);
-                acc = fmaf(__uint_as_float((unsigned)a.acoustic_out[(size_t)r * VT_DIM + c] << 16), xn, acc);
+#pragma unroll
+            for (int i = 0; i < VT_DIM / 512; i++) {
+                const int c = 8 * (lane + 64 * i);
+                const u32x4 w = *reinterpret_cast<const u32x4 *>(a.acoustic_out + (size_t)r * VT_DIM + c);
+                const f32x4 xa = *reinterpret_cast<const f32x4 *>(&s_xn[b][c]);
+                const f32x4 xb = *reinterpret_cast<const f32x4 *>(&s_xn[b][c + 4]);
+                acc = vt_dot8(w, xa, xb, acc);
             }
             acc = vt_wave_sum(acc);
             if (lane == 0) { s_vel[o] = acc; a.vel[o] = acc; }
@@ -317,10 +426,19 @@ vt_ac_edge_kernel(ac_edge_args a) {
     if (a.do_front) {
         /* tokens of both branches: [noise, time, llm] and [noise, time, 0]; the noise token is
          * the 36-term input projection in the CPU order (voxtral_tts_kernels.c:152-185) */
-        for (int c = t; c < VT_DIM; c += 1024) {
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            const int c = t + 1024 * j;
+            const u32x2 *wr = reinterpret_cast<const u32x2 *>(a.input_proj + (size_t)c * VT_AC_DIM_IN);
             float acc = 0.f;
-            for (int k = 0; k < VT_AC_DIM_IN; k++)
-                acc = __fadd_rn(acc, __fmul_rn(__uint_as_float((unsigned)a.input_proj[(size_t)c * VT_AC_DIM_IN + k] << 16), s_x[k]));
+#pragma unroll
+            for (int k4 = 0; k4 < VT_AC_DIM_IN / 4; k4++) {
+                const u32x2 w = wr[k4];
+                acc = __fadd_rn(acc, __fmul_rn(vt_bf16_lo(w.x), s_x[4 * k4]));
+                acc = __fadd_rn(acc, __fmul_rn(vt_bf16_hi(w.x), s_x[4 * k4 + 1]));
+                acc = __fadd_rn(acc, __fmul_rn(vt_bf16_lo(w.y), s_x[4 * k4 + 2]));
+                acc = __fadd_rn(acc, __fmul_rn(vt_bf16_hi(w.y), s_x[4 * k4 + 3]));
+            }
             const float tm = a.time_tok[c];
             a.tok_out[c] = acc;
             a.tok_out[VT_DIM + c] = tm;
@@ -394,7 +512,9 @@ static int launch_phase(const uint16_t *W, const float *in, const float *gain, f
         attr_set = 1;
     }
     ac_phase_args a = {W, in, gain, out};
-    hipLaunchKernelGGL(vt_ac_phase_kernel<PH>, dim3(n_rows / 16), dim3(AC_THREADS), lds, g_vt.stream, a);
+    const int n_units = n_rows / AC_RB;
+    const int grid = n_units < g_vt.n_cu ? n_units : g_vt.n_cu;
+    hipLaunchKernelGGL(vt_ac_phase_kernel<PH>, dim3(grid), dim3(AC_THREADS), lds, g_vt.stream, a, n_units);
     return 0;
 }
 
