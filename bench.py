@@ -100,11 +100,220 @@ def cpu_baseline(layers, final_norm, kv_k, kv_v, kv_max, embeds, gpu_hidden, bud
         "steps_checked": len(errs), "against": kind}
 
 
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+LAYER_WEIGHT_ELEMS = LAYER_WEIGHT_BYTES // 2
+PREFILL_LEN = 512
+GEMM_SHAPES = (("q|k|v", 6144, 3072), ("output", 3072, 4096), ("gate|up", 18432, 3072), ("down", 3072, 9216))
+
+
+def prefill_flops(seq):
+    """Algorithmic flops of a 26-layer prefill: 2 M N K per projection plus the causal
+    attention (QK^T and PV over the visible keys of each query, 32 heads of 128)."""
+    gemm = 2 * seq * LAYER_WEIGHT_ELEMS * N_LAYERS
+    attn = 4 * S.HEAD_DIM * S.HEADS * (seq * (seq + 1) // 2) * N_LAYERS
+    return gemm, attn
+
+
+def bench_prefill(args):
+    """BASELINE.json config "Backbone prefill": 26 layers, 512 random token ids, causal GQA
+    attention.  A step is one whole prefill into an empty cache; inputs are resident in HBM."""
+    import cases
+    K, W = args.steps, args.warmup
+    workers = min(16, os.cpu_count() or 8)
+    t0 = time.time()
+    layers = make_layers(N_LAYERS, workers)
+    final_norm = S.norm_weight(S.DIM, 99)
+    ids = np.random.default_rng(11).integers(0, 131072, PREFILL_LEN)
+    with ThreadPoolExecutor(workers) as ex:
+        embeds = np.stack(list(ex.map(emb_row, ids))).astype(np.float32)
+    t_gen = time.time() - t0
+    hip = H.Hip(kv_max=PREFILL_LEN + 8)
+    lib = hip.lib
+    t0 = time.time()
+    hip.upload_decoder(layers, final_norm, N_LAYERS)
+    t_up = time.time() - t0
+    d_e = H.DevBuf.from_numpy(lib, embeds)
+    for _ in range(W):
+        lib.tts_hip_llm_prefill(d_e.ptr, PREFILL_LEN, 0)
+    lib.tts_hip_sync()
+    lib.tts_hip_timer_start()
+    for _ in range(K):
+        lib.tts_hip_llm_prefill(d_e.ptr, PREFILL_LEN, 0)
+    ms_step = lib.tts_hip_timer_stop_ms() / K
+    lib.tts_hip_sync()
+    hip.check()
+    gemm_fl, attn_fl = prefill_flops(PREFILL_LEN)
+    # the dominant kernel alone, per projection shape, timed by the library with events
+    per_shape = {}
+    for i, (name, n, k) in enumerate(GEMM_SHAPES):
+        ms = lib.tts_hip_bench_kernel(i, 50)
+        fl = 2.0 * PREFILL_LEN * n * k
+        per_shape[name] = {"N": n, "K": k, "us": round(ms * 1e3, 1), "tflops": round(fl / ms / 1e9, 1)}
+    ms_attn = lib.tts_hip_bench_kernel(4, 50)
+    hip.check()
+    ms_gemm_layer = sum(v["us"] for v in per_shape.values()) / 1e3
+    achieved = 2.0 * PREFILL_LEN * LAYER_WEIGHT_ELEMS / ms_gemm_layer / 1e9
+    out = {
+        "metric": "backbone prefill ms (512 tokens, 26 layers)",
+        "value": round(ms_step, 4), "unit": "ms/prefill",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 weights x (hi, lo) bf16 activation planes, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "26-layer backbone prefill of 512 random token ids, causal GQA attention "
+                               "(BASELINE.json configs[3])",
+                   "layers": N_LAYERS, "seq_len": PREFILL_LEN, "weights": "bf16 N(0,0.02) seeded, truncated"},
+        "tokens_per_s": round(PREFILL_LEN / (ms_step * 1e-3), 1),
+        "tflops": round((gemm_fl + attn_fl) / ms_step / 1e9, 1),
+        "roofline": {
+            "kernel": "vt_gemm_mfma_kernel (the four projection launches of one layer at M = 512)",
+            "bound": "mfma",
+            "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+            "traffic": None,
+            "flops_per_layer": 2 * PREFILL_LEN * LAYER_WEIGHT_ELEMS,
+            "ms_per_layer": round(ms_gemm_layer, 4),
+            "executed_over_algorithmic": 2.0,
+            "per_shape": per_shape,
+            "attention_us": round(ms_attn * 1e3, 1),
+        },
+        "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
+        "cpu_baseline": None,
+    }
+    if args.cpu_seconds > 0 and S.have_ref():
+        # the reference's own tts_llm_prefill (triple-loop linear, no BLAS in this build), single thread,
+        # on the first n_cpu tokens of the same prompt; the cost per token is flat in this range
+        n_cpu = 2
+        b = cases.RefBackend()
+        b.llm_open(layers, final_norm, 16)
+        t0 = time.time()
+        b.llm_prefill(embeds[:n_cpu])
+        dt = time.time() - t0
+        rk, rv = b.llm_kv()
+        b.llm_close()
+        lib.tts_hip_llm_prefill(embeds[:n_cpu].ctypes.data, n_cpu, 0)
+        gk, gv = hip.kv()
+        errs = [S.rel_errors(rk[l, r], gk[l, r]) for l in (0, N_LAYERS - 1) for r in range(n_cpu)]
+        errs += [S.rel_errors(rv[l, r], gv[l, r]) for l in (0, N_LAYERS - 1) for r in range(n_cpu)]
+        out["cpu_baseline"] = {
+            "value": round(dt / n_cpu * PREFILL_LEN * 1e3, 1), "unit": "ms/prefill", "cores": 1, "kind": "reference",
+            "sample": f"tts_llm_prefill of the first {n_cpu} tokens through all 26 layers ({dt:.1f} s), scaled "
+                      f"linearly to 512 tokens; no-BLAS build of the reference",
+        }
+        out["parity"] = {"max_abs_over_rms": float(f"{max(e[0] for e in errs):.3e}"),
+                         "rel_l2": float(f"{max(e[1] for e in errs):.3e}"),
+                         "checked": f"K and V rows 0..{n_cpu - 1} of layers 0 and 25", "against": "reference"}
+        assert out["parity"]["max_abs_over_rms"] < 1e-3, out["parity"]
+    hip.close()
+    print(json.dumps(out))
+
+
+AC_LAYER_BYTES = LAYER_WEIGHT_BYTES
+AC_PHASES = (("q|k|v", 10, 2 * 6144 * 3072), ("attention+output", 11, 2 * 3072 * 4096),
+             ("gate|up", 12, 2 * 18432 * 3072), ("down", 13, 2 * 3072 * 9216))
+
+
+def acoustic_frame_bytes():
+    """Algorithmic HBM bytes of one frame: 7 Euler steps x 3 layers of bf16 weights (each streamed
+    once per step for both guidance branches), the 36-wide in/out projections per step, the semantic
+    head and the LLM-token projection once per frame.  Time tokens are cached per upload."""
+    per_step = 3 * AC_LAYER_BYTES + 2 * (S.DIM * S.ACOUSTIC_DIM * 2) + 6 * S.DIM * 4
+    return 7 * per_step + 8320 * S.DIM * 2 + S.DIM * S.DIM * 2
+
+
+def bench_acoustic(args):
+    """BASELINE.json config "Flow-matching acoustic transformer per frame": 3 layers, batch 2
+    (conditional + unconditional, guidance 1.2), 7 Euler steps, FSQ.  A step is one frame."""
+    import cases
+    K, W = args.steps, args.warmup
+    t0 = time.time()
+    ac = S.Acoustic(50)
+    t_gen = time.time() - t0
+    hip = H.Hip(kv_max=8)
+    lib = hip.lib
+    t0 = time.time()
+    hip.upload_acoustic(ac)
+    t_up = time.time() - t0
+    st = C.c_uint64(0)
+    S.oracle().orc_rng_seed(C.byref(st), 42)
+    hs, xs = [], []
+    for f in range(8):
+        hs.append(S.f32_normal(S.DIM, 20 + f))
+        x0 = np.zeros(S.ACOUSTIC_DIM, np.float32)
+        S.oracle().orc_randn_fill(C.byref(st), S.fp(x0), S.ACOUSTIC_DIM)
+        xs.append(x0)
+    codes = np.zeros(S.CODES, np.int32)
+    d_h = [H.DevBuf.from_numpy(lib, h) for h in hs]
+    d_x = [H.DevBuf.from_numpy(lib, x) for x in xs]
+    for i in range(W):
+        lib.tts_hip_acoustic_frame(codes.ctypes.data, d_h[i % 8].ptr, d_x[i % 8].ptr, None)
+    lib.tts_hip_sync()
+    t0 = time.time()
+    for i in range(K):
+        lib.tts_hip_acoustic_frame(codes.ctypes.data, d_h[i % 8].ptr, d_x[i % 8].ptr, None)
+    lib.tts_hip_sync()
+    ms_step = (time.time() - t0) * 1e3 / K          # host clock: every frame ends in a device->host copy
+    hip.check()
+    per_phase = {}
+    for name, which, nbytes in AC_PHASES:
+        ms = lib.tts_hip_bench_kernel(which, 50)
+        per_phase[name] = {"us": round(ms * 1e3, 1), "gbps": round(nbytes / ms / 1e6, 1)}
+    hip.check()
+    ms_layer = sum(v["us"] for v in per_phase.values()) / 1e3
+    achieved = AC_LAYER_BYTES / ms_layer / 1e6
+    fb = acoustic_frame_bytes()
+    out = {
+        "metric": "acoustic transformer ms/frame",
+        "value": round(ms_step, 4), "unit": "ms/frame",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 weights x (hi, lo) bf16 activation planes, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "flow-matching acoustic transformer, one frame: semantic head + 7 Euler steps of "
+                               "3 layers at batch 2 x 3 tokens, guidance 1.2, FSQ (BASELINE.json configs[4])",
+                   "weights": "bf16 N(0,0.02) seeded, truncated", "timed": "host clock over whole frames, "
+                   "inputs resident in HBM, 37 codes copied back per frame"},
+        "frames_per_s": round(1000.0 / ms_step, 1),
+        "hbm_gbps": round(fb / (ms_step * 1e-3) / 1e9, 1),
+        "hbm_frac_of_peak": round(fb / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "roofline": {
+            "kernel": "vt_ac_phase_kernel (the four launches of one layer, 6 activation rows)",
+            "bound": "hbm",
+            "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "bytes_per_layer": AC_LAYER_BYTES, "ms_per_layer": round(ms_layer, 4),
+            "per_phase": per_phase,
+        },
+        "bytes_per_frame": fb,
+        "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
+        "cpu_baseline": None,
+    }
+    if args.cpu_seconds > 0 and S.have_ref():
+        # one frame of the reference's tts_acoustic_forward (14 velocity evaluations), single thread
+        b = cases.RefBackend()
+        b.ac_open(ac)
+        t0 = time.time()
+        rc, _ = b.acoustic_forward(hs[0], seed=42)
+        dt = time.time() - t0
+        b.ac_close()
+        g = np.zeros(S.CODES, np.int32)
+        lib.tts_hip_acoustic_frame(g.ctypes.data, d_h[0].ptr, d_x[0].ptr, None)
+        out["cpu_baseline"] = {"value": round(dt * 1e3, 1), "unit": "ms/frame", "cores": 1, "kind": "reference",
+                               "sample": "one frame of tts_acoustic_forward at seed 42 (same hidden state and noise)"}
+        out["parity"] = {"codes_equal": int(np.sum(g == rc)), "codes": int(S.CODES), "against": "reference"}
+        assert np.array_equal(g, rc), (g, rc)
+    hip.close()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", choices=("decode", "prefill", "acoustic"), default="decode",
+                    help="decode = the headline metric; prefill / acoustic = the other two configurations")
     ap.add_argument("--mode", type=int, default=0, help="0 persistent kernel, 1 per-phase kernels, 2 streaming kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--calibrate", action="store_true",
@@ -117,6 +326,10 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus above 1 is not supported "
                  "(the decode chain is not sharded; see DESIGN.md)")
+    if args.workload == "prefill":
+        return bench_prefill(args)
+    if args.workload == "acoustic":
+        return bench_acoustic(args)
     K, W = args.steps, args.warmup
     workers = min(16, os.cpu_count() or 8)
 

@@ -202,6 +202,12 @@ const char *tts_hip_last_error(void);
 /* Event timing on the internal stream (for benchmarks). */
 void tts_hip_timer_start(void);
 float tts_hip_timer_stop_ms(void);
+/* Average duration in ms of one launch of a single kernel, timed with events on the
+ * internal stream over `iters` launches on zero-filled work buffers (needs the weights
+ * of layer 0 uploaded): which 0..3 = sequence-level product at M = 512 with the q|k|v,
+ * output, gate/up and down projection; 4 = causal attention at 512 queries (KV cache of
+ * at least 512 rows); 10..13 = the four acoustic phase kernels.  Negative on error. */
+float tts_hip_bench_kernel(int which, int iters);
 
 #ifdef __cplusplus
 }

@@ -95,6 +95,7 @@ SIGNATURES = {
     "tts_hip_last_error": (C.c_char_p, []),
     "tts_hip_timer_start": (None, []),
     "tts_hip_timer_stop_ms": (C.c_float, []),
+    "tts_hip_bench_kernel": (C.c_float, [C.c_int, C.c_int]),
 }
 
 _lib = None

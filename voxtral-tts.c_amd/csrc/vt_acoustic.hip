@@ -531,6 +531,31 @@ static int run_layers(const ac_work *w) {
     return 0;
 }
 
+/* average duration (ms) of one launch of phase `phase` of acoustic layer 0 on the work area */
+float vt_bench_acoustic_phase(int phase, int iters) {
+    if (!g_vt.initialized || !g_vt.ac_uploaded) { vt_set_error("bench: acoustic weights not uploaded"); return -1.f; }
+    float *base = (float *)vt_scratch(sizeof(float) * AC_WORK_FLOATS);
+    if (!base) return -1.f;
+    ac_work w;
+    carve(&w, base);
+    if (vt_check(hipMemsetAsync(base, 0, sizeof(float) * AC_WORK_FLOATS, g_vt.stream), "bench clear")) return -1.f;
+    const vt_layer_dev *L = &g_vt.ac.layers[0];
+    float ms = -1.f;
+    for (int it = -2; it < iters; it++) {
+        if (it == 0 && vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench start")) return -1.f;
+        int r = -1;
+        if (phase == AC_QKV) r = launch_phase<AC_QKV>(L->wqkv, w.tok, L->attn_norm, w.qkv, VT_QKV_DIM);
+        if (phase == AC_WO) r = launch_phase<AC_WO>(L->wo, w.qkv, NULL, w.tok, VT_DIM);
+        if (phase == AC_W13) r = launch_phase<AC_W13>(L->w13, w.tok, L->ffn_norm, w.h, 2 * VT_FFN);
+        if (phase == AC_W2) r = launch_phase<AC_W2>(L->w2, w.h, NULL, w.tok, VT_DIM);
+        if (r) return -1.f;
+    }
+    if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;
+    if (vt_check(hipEventSynchronize(g_vt.ev1), "bench sync")) return -1.f;
+    if (vt_check(hipEventElapsedTime(&ms, g_vt.ev0, g_vt.ev1), "bench time")) return -1.f;
+    return ms / (float)iters;
+}
+
 static void launch_edge(const ac_work *w, const float *time_tok, float dt, int back, int euler, int front, int fsq) {
     const vt_acoustic_dev *ac = &g_vt.ac;
     ac_edge_args a;

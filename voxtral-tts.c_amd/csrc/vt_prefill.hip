@@ -306,3 +306,40 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
 extern "C" void tts_hip_llm_prefill(const float *embeds, int seq_len, int start_pos) {
     tts_hip_llm_prefill_out(embeds, seq_len, start_pos, NULL);
 }
+
+/* ---- single-kernel timing for benchmarks ---------------------------------------------
+ * which 0..3: the matrix-core product at M = 512 with the q|k|v, output, gate/up and
+ * down projection of backbone layer 0 (splits as in the prefill); 4: the causal
+ * attention at 512 queries; 10..13: the four acoustic phase kernels of acoustic layer 0.
+ * Returns the average duration of one launch in ms (events on the internal stream), or
+ * a negative value on error.  Buffers hold zeros: the kernels are data-independent. */
+float vt_bench_acoustic_phase(int phase, int iters);
+
+extern "C" float tts_hip_bench_kernel(int which, int iters) {
+    if (!g_vt.initialized || iters < 1) { vt_set_error("tts_hip_bench_kernel: bad call"); return -1.f; }
+    if (which >= 10 && which <= 13) return vt_bench_acoustic_phase(which - 10, iters);
+    if (which < 0 || which > 4 || g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_bench_kernel: unknown kernel %d", which); return -1.f; }
+    const int S = 512;
+    if (which == 4 && g_vt.kv_max < S) { vt_set_error("tts_hip_bench_kernel: KV cache shorter than 512"); return -1.f; }
+    const vt_layer_dev *L = &g_vt.h_layers[0];
+    static const int NN[4] = {VT_QKV_DIM, VT_DIM, 2 * VT_FFN, VT_DIM}, KK[4] = {VT_DIM, VT_Q_DIM, VT_DIM, VT_FFN},
+                     SP[4] = {1, 2, 1, 3};
+    const size_t n_out = (size_t)S * 2 * VT_FFN * 3, n_plane = (size_t)S * VT_FFN, n_q = (size_t)S * VT_Q_DIM;
+    const size_t bytes = sizeof(float) * (n_out + n_q) + 2 * sizeof(uint16_t) * n_plane;
+    unsigned char *base = (unsigned char *)vt_scratch(bytes);
+    if (!base) return -1.f;
+    if (vt_check(hipMemsetAsync(base, 0, bytes, g_vt.stream), "bench clear")) return -1.f;
+    float *out = (float *)base, *q = out + n_out;
+    uint16_t *hi = (uint16_t *)(q + n_q), *lo = hi + n_plane;
+    const uint16_t *W[4] = {L->wqkv, L->wo, L->w13, L->w2};
+    float ms = -1.f;
+    for (int it = -2; it < iters; it++) {
+        if (it == 0 && vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench start")) return -1.f;
+        if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], SP[which]);
+        else vt_launch_prefill_attention(out, NULL, NULL, q, VT_Q_DIM, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu, S, 0);
+    }
+    if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;
+    if (vt_check(hipEventSynchronize(g_vt.ev1), "bench sync")) return -1.f;
+    if (vt_check(hipEventElapsedTime(&ms, g_vt.ev0, g_vt.ev1), "bench time")) return -1.f;
+    return ms / (float)iters;
+}
