@@ -18,15 +18,21 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 /* ---- RoPE + cache append ------------------------------------------------------- */
 
-/* qkv [S,6144] -> q [S,4096] with RoPE, cache rows start_pos.. (k with RoPE, v) */
-__global__ void vt_split_qkv_rope_kernel(const float *qkv, float *q, float *kc, float *vc,
-                                         const float *rope, int start_pos, int S) {
+/* qkv [S,6144] (the sum of `planes` split-K planes, `plane_stride` floats apart) ->
+ * q [S,4096] with RoPE, cache rows start_pos.. (k with RoPE, v) */
+__global__ void vt_split_qkv_rope_kernel(const float *qkv, int planes, size_t plane_stride, float *q,
+                                         float *kc, float *vc, const float *rope, int start_pos, int S) {
     const int pairs = VT_QKV_DIM / 2;
     const size_t total = (size_t)S * pairs;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (size_t)gridDim.x * blockDim.x) {
         const int s = (int)(i / pairs), g = (int)(i % pairs) * 2;
-        const f32x2 ab = *reinterpret_cast<const f32x2 *>(qkv + (size_t)s * VT_QKV_DIM + g);
+        f32x2 ab = *reinterpret_cast<const f32x2 *>(qkv + (size_t)s * VT_QKV_DIM + g);
+        for (int p = 1; p < planes; p++) {
+            const f32x2 w = *reinterpret_cast<const f32x2 *>(qkv + p * plane_stride + (size_t)s * VT_QKV_DIM + g);
+            ab.x = __fadd_rn(ab.x, w.x);
+            ab.y = __fadd_rn(ab.y, w.y);
+        }
         f32x2 o = ab;
         float *dst;
         if (g < VT_Q_DIM + VT_KV_DIM) {
@@ -271,7 +277,11 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
     const size_t S = (size_t)seq_len;
     hipStream_t st = g_vt.stream;
     /* work area: x | wide f32 (qkv or gate/up) | q | partial planes | hi | lo */
-    const size_t n_x = S * VT_DIM, n_wide = S * 2 * VT_FFN, n_q = S * VT_Q_DIM, n_part = 3 * S * VT_DIM;
+    /* K is cut so that every product launches about two workgroups per CU (M tiles x N tiles x
+     * cuts): 4 M tiles at 512 rows give 192 / 96 / 96 tiles for q|k|v / output / down */
+    const int m_tiles = (seq_len + 127) / 128;
+    const int sp_qkv = m_tiles >= 3 ? 2 : 4, sp_wo = m_tiles >= 3 ? 4 : 8, sp_w2 = m_tiles >= 3 ? 4 : 8;
+    const size_t n_x = S * VT_DIM, n_wide = S * 4 * VT_QKV_DIM, n_q = S * VT_Q_DIM, n_part = 8 * S * VT_DIM;
     const size_t n_plane = S * VT_FFN;                            /* bf16 elements per plane */
     const size_t bytes = sizeof(float) * (n_x + n_wide + n_q + n_part) + 2 * sizeof(uint16_t) * n_plane;
     float *x = (float *)vt_scratch(bytes);
@@ -286,17 +296,17 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         const vt_layer_dev *L = &g_vt.h_layers[l];
         float *kc = g_hip.kv_cache_k_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
         float *vc = g_hip.kv_cache_v_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
-        vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, 1);
+        vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
         hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(ew_blocks(S * VT_QKV_DIM / 2)), dim3(256), 0, st,
-                           wide, q, kc, vc, g_vt.d_rope, start_pos, seq_len);
+                           wide, sp_qkv, S * VT_QKV_DIM, q, kc, vc, g_vt.d_rope, start_pos, seq_len);
         vt_launch_prefill_attention(NULL, hi, lo, q, VT_Q_DIM, kc, vc, seq_len, start_pos);
-        vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, 2);
-        vt_launch_residual_norm_split(x, part, 2, ps, L->ffn_norm, hi, lo, seq_len);
+        vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
+        vt_launch_residual_norm_split(x, part, sp_wo, ps, L->ffn_norm, hi, lo, seq_len);
         vt_launch_gemm(wide, hi, lo, L->w13, seq_len, 2 * VT_FFN, VT_DIM, 1);
         vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN);
-        vt_launch_gemm(part, hi, lo, L->w2, seq_len, VT_DIM, VT_FFN, 3);
+        vt_launch_gemm(part, hi, lo, L->w2, seq_len, VT_DIM, VT_FFN, sp_w2);
         const float *next_norm = l + 1 < g_vt.n_dec_layers ? g_vt.h_layers[l + 1].attn_norm : NULL;
-        vt_launch_residual_norm_split(x, part, 3, ps, next_norm, hi, lo, seq_len);
+        vt_launch_residual_norm_split(x, part, sp_w2, ps, next_norm, hi, lo, seq_len);
     }
     VT_TRYV(hipGetLastError());
     VT_TRYV(hipStreamSynchronize(st));
@@ -323,8 +333,8 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
     if (which == 4 && g_vt.kv_max < S) { vt_set_error("tts_hip_bench_kernel: KV cache shorter than 512"); return -1.f; }
     const vt_layer_dev *L = &g_vt.h_layers[0];
     static const int NN[4] = {VT_QKV_DIM, VT_DIM, 2 * VT_FFN, VT_DIM}, KK[4] = {VT_DIM, VT_Q_DIM, VT_DIM, VT_FFN},
-                     SP[4] = {1, 2, 1, 3};
-    const size_t n_out = (size_t)S * 2 * VT_FFN * 3, n_plane = (size_t)S * VT_FFN, n_q = (size_t)S * VT_Q_DIM;
+                     SP[4] = {2, 4, 1, 4};
+    const size_t n_out = (size_t)S * 2 * VT_FFN * 4, n_plane = (size_t)S * VT_FFN, n_q = (size_t)S * VT_Q_DIM;
     const size_t bytes = sizeof(float) * (n_out + n_q) + 2 * sizeof(uint16_t) * n_plane;
     unsigned char *base = (unsigned char *)vt_scratch(bytes);
     if (!base) return -1.f;
