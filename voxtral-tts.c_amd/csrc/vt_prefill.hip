@@ -14,7 +14,6 @@
 
 #include <math.h>
 
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 /* ---- RoPE + cache append ------------------------------------------------------- */
 
@@ -50,71 +49,77 @@ __global__ void vt_split_qkv_rope_kernel(const float *qkv, int planes, size_t pl
     }
 }
 
-/* ---- causal attention, 32 queries x 32 keys per matrix-core tile --------------
+/* ---- causal attention, 16 queries x 32 keys per matrix-core tile ----------------
  * (tts_causal_attention, voxtral_tts_kernels.c:403-465, for head_dim 128 and four
  * query heads per KV head.)
  *
- * Workgroup = (KV head, block of 32 queries), 4*NSPLIT waves: wave = (query head
- * of the group, key-tile residue).  The waves of one residue share 32-key K and V
- * tiles in LDS.  Scores are computed transposed, S^T = K Q^T, with
- * v_mfma_f32_32x32x2_f32, so that a lane owns one query: lane l holds query l%32
- * and the keys 8*(v/4) + 4*(l/32) + v%4 of the tile in accumulator element v.
- * The softmax state is then per lane (one exchange with lane l^32 per tile), and
- * the probabilities are already in the operand layout of the second product
+ * Workgroup = (KV head, HPW of its 4 query heads, block of 16 queries), HPW*NSPLIT
+ * waves: wave = (query head, key-tile residue).  The waves of one residue share 32-key
+ * K and V tiles in LDS.  Scores are computed transposed, S^T = K Q^T, with
+ * v_mfma_f32_16x16x4_f32, so that a lane owns one query: lane l holds query l%16 and
+ * the keys 4*(l/16) + v of each 16-key block in accumulator element v.  The softmax
+ * state is then per lane (two exchanges across the four lane groups per tile), and the
+ * probabilities are already in the operand layout of the second product
  * O^T = V^T P^T, whose reduction index runs over the keys in that same order.
- * fp32 operands throughout.  Residues are merged through LDS at the end. */
-#define PA_KP 132                 /* K tile pitch in floats: 16-byte reads over keys cover all banks */
-#define PA_VP 136                 /* V tile pitch: lanes l and l^32 (4 keys apart) use disjoint banks */
-#define PA_TILE_FLOATS (32 * PA_KP + 32 * PA_VP)
+ * fp32 operands throughout.  Residues are merged through LDS at the end.
+ * 16-query blocks give 32 blocks per KV head at 512 queries: with HPW = 2 that is 512
+ * workgroups whose work grows with the block index (causal), enough to keep 256 CUs
+ * busy when long and short blocks follow each other. */
+#define PA_QT 16                  /* queries per workgroup */
+#define PA_KP 132                 /* tile pitch in floats: 16-byte reads over 16 keys cover all banks,
+                                     and rows 4 apart (the lane groups of the P V operand) do not collide */
+#define PA_TILE_FLOATS (2 * 32 * PA_KP)
 
-template <int NSPLIT>
-__global__ void __launch_bounds__(256 * NSPLIT)
+template <int NSPLIT, int HPW>
+__global__ void __launch_bounds__(64 * HPW * NSPLIT)
 vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, const float *Q,
                             int q_stride, const float *Kc, const float *Vc, int S,
                             int start_pos, float scale) {
     extern __shared__ __attribute__((aligned(16))) float pa_lds[];
-    const int g = (int)blockIdx.x, qt = (int)blockIdx.y;
+    constexpr int GT = 64 * HPW;                         /* threads of a residue group */
+    constexpr int NLD = 1024 / GT;                       /* 16-byte loads per thread and tile */
+    const int kvh = (int)blockIdx.x / (4 / HPW), hsub = (int)blockIdx.x % (4 / HPW);
+    /* long blocks first: the last query block has the most keys */
+    const int qt = (int)gridDim.y - 1 - (int)blockIdx.y;
     const int t = (int)threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int hq = wave & 3, pz = wave >> 2;
-    const int tl = (hq << 6) | lane;                     /* thread index inside the residue group */
-    const int hh = lane >> 5, qi = lane & 31;
-    const int q0 = qt * 32;
-    const int my_q = q0 + qi;
-    const int head = g * 4 + hq;
+    const int hq = wave % HPW, pz = wave / HPW;
+    const int tl = hq * 64 + lane;                       /* thread index inside the residue group */
+    const int g = lane >> 4, li = lane & 15;
+    const int q0 = qt * PA_QT;
+    const int my_q = q0 + li;
+    const int head = kvh * 4 + hsub * HPW + hq;
     float *Kt = pa_lds + (size_t)pz * PA_TILE_FLOATS, *Vt = Kt + 32 * PA_KP;
 
-    /* this lane's query: dims 64*hh .. 64*hh+63 */
-    float qreg[64];
+    /* this lane's query: dims 32*g .. 32*g+31 */
+    float qreg[32];
     {
-        const float *qp = Q + (size_t)(my_q < S ? my_q : S - 1) * q_stride + head * VT_HEAD_DIM + 64 * hh;
+        const float *qp = Q + (size_t)(my_q < S ? my_q : S - 1) * q_stride + head * VT_HEAD_DIM + 32 * g;
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
+        for (int i = 0; i < 8; i++) {
             const f32x4 v = reinterpret_cast<const f32x4 *>(qp)[i];
             qreg[4 * i] = v.x; qreg[4 * i + 1] = v.y; qreg[4 * i + 2] = v.z; qreg[4 * i + 3] = v.w;
         }
     }
-    f32x16 o[4];
+    f32x4 o[8];
 #pragma unroll
-    for (int b = 0; b < 4; b++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) o[b][v] = 0.f;
+    for (int b = 0; b < 8; b++) o[b] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m = -1e30f, lsum = 0.f;
 
-    const int last_q = (q0 + 31 < S ? q0 + 31 : S - 1) + start_pos;
+    const int last_q = (q0 + PA_QT - 1 < S ? q0 + PA_QT - 1 : S - 1) + start_pos;
     const int ntiles = last_q / 32 + 1;                  /* key tiles 0 .. ntiles-1 are visible */
     const int nsteps = (ntiles + NSPLIT - 1) / NSPLIT;
     const int kv_rows = start_pos + S;
 
-    /* staging: the 256 threads of a residue group move 32 rows x 512 B of K and of V */
-    f32x4 rk[4], rv[4];
+    /* staging: the threads of a residue group move 32 rows x 512 B of K and of V */
+    f32x4 rk[NLD], rv[NLD];
     auto fetch = [&](int tile) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int c = tl + 256 * i, row = c >> 5, col = (c & 31) * 4;
+        for (int i = 0; i < NLD; i++) {
+            const int c = tl + GT * i, row = c >> 5, col = (c & 31) * 4;
             int kr = tile * 32 + row;
             if (kr >= kv_rows) kr = kv_rows - 1;
-            rk[i] = *reinterpret_cast<const f32x4 *>(Kc + (size_t)kr * VT_KV_DIM + g * VT_HEAD_DIM + col);
-            rv[i] = *reinterpret_cast<const f32x4 *>(Vc + (size_t)kr * VT_KV_DIM + g * VT_HEAD_DIM + col);
+            rk[i] = *reinterpret_cast<const f32x4 *>(Kc + (size_t)kr * VT_KV_DIM + kvh * VT_HEAD_DIM + col);
+            rv[i] = *reinterpret_cast<const f32x4 *>(Vc + (size_t)kr * VT_KV_DIM + kvh * VT_HEAD_DIM + col);
         }
     };
     if (pz < ntiles) fetch(pz);
@@ -125,75 +130,82 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
         __syncthreads();
         if (valid) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int c = tl + 256 * i, row = c >> 5, col = (c & 31) * 4;
+            for (int i = 0; i < NLD; i++) {
+                const int c = tl + GT * i, row = c >> 5, col = (c & 31) * 4;
                 *reinterpret_cast<f32x4 *>(Kt + row * PA_KP + col) = rk[i];
-                *reinterpret_cast<f32x4 *>(Vt + row * PA_VP + col) = rv[i];
+                *reinterpret_cast<f32x4 *>(Vt + row * PA_KP + col) = rv[i];
             }
         }
         __syncthreads();
         if (tile + NSPLIT < ntiles) fetch(tile + NSPLIT);
         if (!valid) continue;
 
-        /* S^T = K Q^T over d = 64*hh + ks */
-        f32x16 s;
+        /* S^T = K Q^T: reduction step (j, e) pairs dim 32*g + 4*j + e of key and query */
+        f32x4 s[2];
 #pragma unroll
-        for (int v = 0; v < 16; v++) s[v] = 0.f;
+        for (int kb = 0; kb < 2; kb++) {
+            s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int gk = 0; gk < 16; gk++) {
-            const f32x4 kf = *reinterpret_cast<const f32x4 *>(Kt + qi * PA_KP + 64 * hh + 4 * gk);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.x, qreg[4 * gk], s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.y, qreg[4 * gk + 1], s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.z, qreg[4 * gk + 2], s, 0, 0, 0);
-            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kf.w, qreg[4 * gk + 3], s, 0, 0, 0);
+            for (int j = 0; j < 8; j++) {
+                const f32x4 kf = *reinterpret_cast<const f32x4 *>(Kt + (16 * kb + li) * PA_KP + 32 * g + 4 * j);
+                s[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.x, qreg[4 * j], s[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.y, qreg[4 * j + 1], s[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.z, qreg[4 * j + 2], s[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.w, qreg[4 * j + 3], s[kb], 0, 0, 0);
+            }
         }
-        /* online softmax for this lane's query */
+        /* online softmax for this lane's query; element v of block kb is key 16*kb + 4*g + v */
         const int qpos = start_pos + my_q;
         float mx = -1e30f;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const int kpos = tile * 32 + 8 * (v >> 2) + 4 * hh + (v & 3);
-            s[v] = kpos <= qpos ? __fmul_rn(s[v], scale) : -3e38f;
-            mx = fmaxf(mx, s[v]);
-        }
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int kpos = tile * 32 + 16 * kb + 4 * g + v;
+                s[kb][v] = kpos <= qpos ? __fmul_rn(s[kb][v], scale) : -3e38f;
+                mx = fmaxf(mx, s[kb][v]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float mn = fmaxf(m, mx);
         const float corr = __expf(m - mn);
         float psum = 0.f;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            s[v] = s[v] > -1e38f ? __expf(s[v] - mn) : 0.f;
-            psum += s[v];
-        }
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                s[kb][v] = s[kb][v] > -1e38f ? __expf(s[kb][v] - mn) : 0.f;
+                psum += s[kb][v];
+            }
         lsum = fmaf(lsum, corr, psum);
         m = mn;
 #pragma unroll
-        for (int b = 0; b < 4; b++)
+        for (int b = 0; b < 8; b++) o[b] = o[b] * corr;
+        /* O^T += V^T P^T: reduction step (kb, v) pairs key 16*kb + 4*g + v with s[kb][v] */
 #pragma unroll
-            for (int v = 0; v < 16; v++) o[b][v] *= corr;
-        /* O^T += V^T P^T: reduction step ks pairs key 8*(ks/4) + 4*hh + ks%4 with s[ks] */
+        for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-        for (int ks = 0; ks < 16; ks++) {
-            const float *vrow = Vt + (8 * (ks >> 2) + 4 * hh + (ks & 3)) * PA_VP + qi;
+            for (int v = 0; v < 4; v++) {
+                const float *vrow = Vt + (16 * kb + 4 * g + v) * PA_KP + li;
 #pragma unroll
-            for (int b = 0; b < 4; b++)
-                o[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * b], s[ks], o[b], 0, 0, 0);
-        }
+                for (int b = 0; b < 8; b++)
+                    o[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(vrow[16 * b], s[kb][v], o[b], 0, 0, 0);
+            }
     }
 
     /* merge the residues: residue r > 0 parks (m, l, O) in LDS, residue 0 folds them in */
     if (NSPLIT > 1) {
         __syncthreads();
-        float *park = pa_lds;                            /* [NSPLIT-1][4 heads][66][64 lanes] */
+        float *park = pa_lds;                            /* [NSPLIT-1][HPW][34][64 lanes] */
         for (int r = 1; r < NSPLIT; r++) {
-            float *slot = park + ((size_t)((r - 1) * 4 + hq) * 66) * 64 + lane;
+            float *slot = park + ((size_t)((r - 1) * HPW + hq) * 34) * 64 + lane;
             if (pz == r) {
                 slot[0] = m;
                 slot[64] = lsum;
 #pragma unroll
-                for (int b = 0; b < 4; b++)
+                for (int b = 0; b < 8; b++)
 #pragma unroll
-                    for (int v = 0; v < 16; v++) slot[(2 + b * 16 + v) * 64] = o[b][v];
+                    for (int v = 0; v < 4; v++) slot[(2 + b * 4 + v) * 64] = o[b][v];
             }
             __syncthreads();
             if (pz == 0) {
@@ -203,46 +215,46 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
                 lsum = fmaf(lsum, c1, l2 * c2);
                 m = mn;
 #pragma unroll
-                for (int b = 0; b < 4; b++)
+                for (int b = 0; b < 8; b++)
 #pragma unroll
-                    for (int v = 0; v < 16; v++) o[b][v] = fmaf(o[b][v], c1, slot[(2 + b * 16 + v) * 64] * c2);
+                    for (int v = 0; v < 4; v++) o[b][v] = fmaf(o[b][v], c1, slot[(2 + b * 4 + v) * 64] * c2);
             }
             __syncthreads();
         }
     }
     if (pz != 0 || my_q >= S) return;
-    const float L = lsum + __shfl_xor(lsum, 32);
+    float L = lsum + __shfl_xor(lsum, 16);
+    L += __shfl_xor(L, 32);
     const float inv = L > 0.f ? __fdiv_rn(1.0f, L) : 0.f;
     const size_t ob = (size_t)my_q * VT_Q_DIM + head * VT_HEAD_DIM;
 #pragma unroll
-    for (int b = 0; b < 4; b++)
-#pragma unroll
-        for (int v4 = 0; v4 < 4; v4++) {
-            const int d = 32 * b + 8 * v4 + 4 * hh;
-            f32x4 r;
-            r.x = __fmul_rn(o[b][4 * v4], inv);
-            r.y = __fmul_rn(o[b][4 * v4 + 1], inv);
-            r.z = __fmul_rn(o[b][4 * v4 + 2], inv);
-            r.w = __fmul_rn(o[b][4 * v4 + 3], inv);
-            if (out) *reinterpret_cast<f32x4 *>(out + ob + d) = r;
-            if (out_hi) {
-                unsigned h0, l0, h1, l1, h2, l2, h3, l3;
-                vt_split_planes(r.x, h0, l0);
-                vt_split_planes(r.y, h1, l1);
-                vt_split_planes(r.z, h2, l2);
-                vt_split_planes(r.w, h3, l3);
-                u32x2 ph = {h0 | (h1 << 16), h2 | (h3 << 16)}, pl = {l0 | (l1 << 16), l2 | (l3 << 16)};
-                *reinterpret_cast<u32x2 *>(out_hi + ob + d) = ph;
-                *reinterpret_cast<u32x2 *>(out_lo + ob + d) = pl;
-            }
+    for (int b = 0; b < 8; b++) {
+        const int d = 16 * b + 4 * g;
+        f32x4 r;
+        r.x = __fmul_rn(o[b][0], inv);
+        r.y = __fmul_rn(o[b][1], inv);
+        r.z = __fmul_rn(o[b][2], inv);
+        r.w = __fmul_rn(o[b][3], inv);
+        if (out) *reinterpret_cast<f32x4 *>(out + ob + d) = r;
+        if (out_hi) {
+            unsigned h0, l0, h1, l1, h2, l2, h3, l3;
+            vt_split_planes(r.x, h0, l0);
+            vt_split_planes(r.y, h1, l1);
+            vt_split_planes(r.z, h2, l2);
+            vt_split_planes(r.w, h3, l3);
+            u32x2 ph = {h0 | (h1 << 16), h2 | (h3 << 16)}, pl = {l0 | (l1 << 16), l2 | (l3 << 16)};
+            *reinterpret_cast<u32x2 *>(out_hi + ob + d) = ph;
+            *reinterpret_cast<u32x2 *>(out_lo + ob + d) = pl;
         }
+    }
 }
 
 #define PA_NSPLIT 2
+#define PA_HPW 2
 
-static size_t pa_lds_bytes(int nsplit) {
-    size_t tiles = sizeof(float) * (size_t)nsplit * PA_TILE_FLOATS;
-    size_t park = sizeof(float) * (size_t)(nsplit - 1) * 4 * 66 * 64;
+static size_t pa_lds_bytes(void) {
+    size_t tiles = sizeof(float) * (size_t)PA_NSPLIT * PA_TILE_FLOATS;
+    size_t park = sizeof(float) * (size_t)(PA_NSPLIT - 1) * PA_HPW * 34 * 64;
     return tiles > park ? tiles : park;
 }
 
@@ -252,15 +264,16 @@ void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, c
     const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
     static int attr_set = 0;
     if (!attr_set) {
-        if (vt_check(hipFuncSetAttribute((const void *)vt_prefill_attention_kernel<PA_NSPLIT>,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)pa_lds_bytes(PA_NSPLIT)), "attention LDS size"))
+        if (vt_check(hipFuncSetAttribute((const void *)vt_prefill_attention_kernel<PA_NSPLIT, PA_HPW>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)pa_lds_bytes()),
+                     "attention LDS size"))
             return;
         attr_set = 1;
     }
-    hipLaunchKernelGGL(vt_prefill_attention_kernel<PA_NSPLIT>, dim3(VT_KV_HEADS, (S + 31) / 32),
-                       dim3(256 * PA_NSPLIT), pa_lds_bytes(PA_NSPLIT), g_vt.stream, d_out, d_hi, d_lo, d_Q,
-                       q_stride, d_K, d_V, S, start_pos, scale);
+    hipLaunchKernelGGL((vt_prefill_attention_kernel<PA_NSPLIT, PA_HPW>),
+                       dim3(VT_KV_HEADS * (4 / PA_HPW), (S + PA_QT - 1) / PA_QT), dim3(64 * PA_HPW * PA_NSPLIT),
+                       pa_lds_bytes(), g_vt.stream, d_out, d_hi, d_lo, d_Q, q_stride, d_K, d_V, S, start_pos,
+                       scale);
 }
 
 /* ---- backbone prefill ------------------------------------------------------------ */
