@@ -13,13 +13,17 @@ int vt_gemm_shape_ok(int M, int N, int K, int splits);
 /* d_C: `splits` planes of [M, N] fp32, plane s holds the sum over K range s */
 void vt_launch_gemm(float *d_C, const uint16_t *d_Ahi, const uint16_t *d_Alo, const uint16_t *d_W,
                     int M, int N, int K, int splits);
+/* the same with the row pitch of C and the distance between planes given */
+void vt_launch_gemm_ex(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
+                       const uint16_t *d_W, int M, int N, int K, int splits);
 /* n even */
 void vt_launch_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_x, size_t n);
 /* rows of 3072: x += sum of planes (splits > 0), then planes of rmsnorm(x)*w (d_w != NULL) */
 void vt_launch_residual_norm_split(float *d_x, const float *d_part, int splits, size_t part_stride,
                                    const float *d_w, uint16_t *d_hi, uint16_t *d_lo, int rows);
 /* n_out even: planes of silu(gate)*up from interleaved (gate, up) pairs */
-void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, size_t n_out);
+void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, size_t n_out, int tail_col0,
+                            const float *d_tail, int tail_planes, size_t tail_stride);
 void vt_launch_sum_planes(float *d_out, const float *d_part, int splits, size_t stride, size_t n);
 
 #endif /* VT_GEMM_H */

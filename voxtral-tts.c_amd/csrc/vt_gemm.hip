@@ -42,7 +42,7 @@ __device__ __forceinline__ bf16x8 gm_frag(const unsigned char *p) {
 
 __global__ void __launch_bounds__(256, 2)
 vt_gemm_mfma_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const uint16_t *W,
-                    int M, int N, int K, int k_split, int m_tiles, int n_tiles) {
+                    int M, int N, int K, int k_split, int m_tiles, int n_tiles, int ldc, size_t plane_stride) {
     __shared__ __attribute__((aligned(16))) unsigned char lds[3 * GM_MAT];
     const int id = (int)blockIdx.x;
     int mt, nt, sp;
@@ -141,7 +141,7 @@ vt_gemm_mfma_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const ui
     }
 
     /* accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 */
-    float *Cs = C + (size_t)sp * M * N;
+    float *Cs = C + (size_t)sp * plane_stride;
 #pragma unroll
     for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -150,7 +150,7 @@ vt_gemm_mfma_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const ui
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int row = mt * GM_TILE + 64 * wm + 32 * a + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (row < M) Cs[(size_t)row * N + col] = acc[a][b][v];
+                if (row < M) Cs[(size_t)row * ldc + col] = acc[a][b][v];
             }
         }
 }
@@ -159,11 +159,16 @@ int vt_gemm_shape_ok(int M, int N, int K, int splits) {
     return M >= 1 && splits >= 1 && N % GM_TILE == 0 && K % splits == 0 && (K / splits) % GM_BK == 0;
 }
 
-void vt_launch_gemm(float *d_C, const uint16_t *d_Ahi, const uint16_t *d_Alo, const uint16_t *d_W,
-                    int M, int N, int K, int splits) {
+void vt_launch_gemm_ex(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
+                       const uint16_t *d_W, int M, int N, int K, int splits) {
     const int m_tiles = (M + GM_TILE - 1) / GM_TILE, n_tiles = N / GM_TILE;
     hipLaunchKernelGGL(vt_gemm_mfma_kernel, dim3(m_tiles * n_tiles * splits), dim3(256), 0, g_vt.stream,
-                       d_C, d_Ahi, d_Alo, d_W, M, N, K, K / splits, m_tiles, n_tiles);
+                       d_C, d_Ahi, d_Alo, d_W, M, N, K, K / splits, m_tiles, n_tiles, ldc, plane_stride);
+}
+
+void vt_launch_gemm(float *d_C, const uint16_t *d_Ahi, const uint16_t *d_Alo, const uint16_t *d_W,
+                    int M, int N, int K, int splits) {
+    vt_launch_gemm_ex(d_C, N, (size_t)M * N, d_Ahi, d_Alo, d_W, M, N, K, splits);
 }
 
 /* ---- fp32 -> (hi, lo) bf16 planes ---------------------------------------------- */
@@ -234,11 +239,28 @@ void vt_launch_residual_norm_split(float *d_x, const float *d_part, int splits, 
 }
 
 /* gu [rows, 2*ffn] with (gate, up) adjacent -> (hi, lo) planes of silu(gate)*up
- * (voxtral_tts_llm.c:346-350 on the row-interleaved gate/up matrix). */
-__global__ void vt_swiglu_split_kernel(uint16_t *hi, uint16_t *lo, const float *gu, size_t n2) {
+ * (voxtral_tts_llm.c:346-350 on the row-interleaved gate/up matrix).  Columns from
+ * tail_col0 on are taken as the sum of `tail_planes` split-K planes [rows, 2*ffn - tail_col0]
+ * instead (tail_planes == 0: everything is in gu). */
+__global__ void vt_swiglu_split_kernel(uint16_t *hi, uint16_t *lo, const float *gu, size_t n2,
+                                       int tail_col0, const float *tail, int tail_planes, size_t tail_stride) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n2;
          i += (size_t)gridDim.x * blockDim.x) {
-        const f32x4 g = reinterpret_cast<const f32x4 *>(gu)[i];
+        f32x4 g = reinterpret_cast<const f32x4 *>(gu)[i];
+        if (tail_planes > 0) {
+            const size_t row = (4 * i) / (2 * VT_FFN);
+            const int col = (int)((4 * i) % (2 * VT_FFN));
+            if (col >= tail_col0) {
+                const int tw = 2 * VT_FFN - tail_col0;
+                const float *tp = tail + row * tw + (col - tail_col0);
+                g = *reinterpret_cast<const f32x4 *>(tp);
+                for (int p = 1; p < tail_planes; p++) {
+                    const f32x4 w = *reinterpret_cast<const f32x4 *>(tp + p * tail_stride);
+                    g.x = __fadd_rn(g.x, w.x); g.y = __fadd_rn(g.y, w.y);
+                    g.z = __fadd_rn(g.z, w.z); g.w = __fadd_rn(g.w, w.w);
+                }
+            }
+        }
         const float a = __fmul_rn(__fdiv_rn(g.x, __fadd_rn(1.0f, expf(-g.x))), g.y);
         const float b = __fmul_rn(__fdiv_rn(g.z, __fadd_rn(1.0f, expf(-g.z))), g.w);
         unsigned h0, l0, h1, l1;
@@ -249,9 +271,10 @@ __global__ void vt_swiglu_split_kernel(uint16_t *hi, uint16_t *lo, const float *
     }
 }
 
-void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, size_t n_out) {
+void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, size_t n_out, int tail_col0,
+                            const float *d_tail, int tail_planes, size_t tail_stride) {
     hipLaunchKernelGGL(vt_swiglu_split_kernel, dim3(gm_blocks(n_out / 2)), dim3(256), 0, g_vt.stream, d_hi, d_lo,
-                       d_gu, n_out / 2);
+                       d_gu, n_out / 2, tail_col0, d_tail, tail_planes, tail_stride);
 }
 
 /* C = sum of `splits` partial planes (fixed order), for callers that want the plain product. */

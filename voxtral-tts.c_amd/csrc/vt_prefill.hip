@@ -294,6 +294,7 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
      * cuts): 4 M tiles at 512 rows give 192 / 96 / 96 tiles for q|k|v / output / down */
     const int m_tiles = (seq_len + 127) / 128;
     const int sp_qkv = m_tiles >= 3 ? 2 : 4, sp_wo = m_tiles >= 3 ? 4 : 8, sp_w2 = m_tiles >= 3 ? 4 : 8;
+    const int tail_cols = m_tiles == 4 ? 16 * 128 : 0;      /* part holds 4 x S x 2048 <= 8 x S x 3072 */
     const size_t n_x = S * VT_DIM, n_wide = S * 4 * VT_QKV_DIM, n_q = S * VT_Q_DIM, n_part = 8 * S * VT_DIM;
     const size_t n_plane = S * VT_FFN;                            /* bf16 elements per plane */
     const size_t bytes = sizeof(float) * (n_x + n_wide + n_q + n_part) + 2 * sizeof(uint16_t) * n_plane;
@@ -315,8 +316,18 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         vt_launch_prefill_attention(NULL, hi, lo, q, VT_Q_DIM, kc, vc, seq_len, start_pos);
         vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
         vt_launch_residual_norm_split(x, part, sp_wo, ps, L->ffn_norm, hi, lo, seq_len);
-        vt_launch_gemm(wide, hi, lo, L->w13, seq_len, 2 * VT_FFN, VT_DIM, 1);
-        vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN);
+        if (tail_cols) {
+            /* 4 M tiles x 144 N tiles are 576 workgroups for 512 slots: the last 16 N tiles get their
+             * K cut in 4 instead of running as a nearly empty second round */
+            const int main_cols = 2 * VT_FFN - tail_cols;
+            vt_launch_gemm_ex(wide, 2 * VT_FFN, 0, hi, lo, L->w13, seq_len, main_cols, VT_DIM, 1);
+            vt_launch_gemm_ex(part, tail_cols, S * tail_cols, hi, lo, L->w13 + (size_t)main_cols * VT_DIM, seq_len,
+                              tail_cols, VT_DIM, 4);
+            vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, main_cols, part, 4, S * tail_cols);
+        } else {
+            vt_launch_gemm(wide, hi, lo, L->w13, seq_len, 2 * VT_FFN, VT_DIM, 1);
+            vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, 0, NULL, 0, 0);
+        }
         vt_launch_gemm(part, hi, lo, L->w2, seq_len, VT_DIM, VT_FFN, sp_w2);
         const float *next_norm = l + 1 < g_vt.n_dec_layers ? g_vt.h_layers[l + 1].attn_norm : NULL;
         vt_launch_residual_norm_split(x, part, sp_w2, ps, next_norm, hi, lo, seq_len);
@@ -358,7 +369,12 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
     float ms = -1.f;
     for (int it = -2; it < iters; it++) {
         if (it == 0 && vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench start")) return -1.f;
-        if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], SP[which]);
+        if (which == 2) {                               /* as in the prefill: main part + K-cut tail */
+            const int tail = 16 * 128, main_cols = 2 * VT_FFN - tail;
+            vt_launch_gemm_ex(out, 2 * VT_FFN, 0, hi, lo, W[2], S, main_cols, VT_DIM, 1);
+            vt_launch_gemm_ex(out + (size_t)S * 2 * VT_FFN, tail, (size_t)S * tail, hi, lo,
+                              W[2] + (size_t)main_cols * VT_DIM, S, tail, VT_DIM, 4);
+        } else if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], SP[which]);
         else vt_launch_prefill_attention(out, NULL, NULL, q, VT_Q_DIM, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu, S, 0);
     }
     if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;
