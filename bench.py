@@ -48,6 +48,17 @@ def step_bytes(pos):
     return w + norms + kv_read + kv_write + io
 
 
+def measured_traffic(workload):
+    """HBM bytes per launch (or per layer) of the dominant kernel as measured with rocprofv3
+    --pmc and recorded under profiles/; None when no measurement is on file."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            e = json.load(f)[workload]
+        return 1024.0 * (e["fetch_kib"] * e["fetch_factor"] + e["write_kib"] * e["write_factor"])
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def emb_row(token_id):
     """Row `token_id` of the synthetic [131072, 3072] bf16 embedding table."""
     return S.bf16_to_f32(S.bf16_normal(S.DIM, 7_000_000 + int(token_id), 1.0))
@@ -170,7 +181,7 @@ def bench_prefill(args):
             "bound": "mfma",
             "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": measured_traffic("prefill"),
             "flops_per_layer": 2 * PREFILL_LEN * LAYER_WEIGHT_ELEMS,
             "ms_per_layer": round(ms_gemm_layer, 4),
             "executed_over_algorithmic": 2.0,
@@ -281,7 +292,7 @@ def bench_acoustic(args):
             "bound": "hbm",
             "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": measured_traffic("acoustic"),
             "bytes_per_layer": AC_LAYER_BYTES, "ms_per_layer": round(ms_layer, 4),
             "per_phase": per_phase,
         },
@@ -417,7 +428,7 @@ def main():
     avg_pos = pos0 + (K - 1) / 2.0
     bytes_launch = step_bytes(avg_pos)
     achieved = bytes_launch / (ms_kernel * 1e-3) / 1e9
-    traffic = None if args.traffic_kib is None else args.traffic_kib * 1024.0
+    traffic = measured_traffic("decode") if args.traffic_kib is None else args.traffic_kib * 1024.0
     out = {
         "metric": "backbone decode ms/frame",
         "value": round(ms_step, 4),
