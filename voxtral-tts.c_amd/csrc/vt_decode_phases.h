@@ -29,7 +29,7 @@
 
 #define VT_RING 18            /* 16-byte buffers per lane in the row ring */
 #define VT_ATT_STRIDE 132     /* floats per attention partial: m, l, pad, pad, o[128] */
-#define VT_ATT_MIN_CHUNK 128  /* positions per attention workgroup before the cache is split further */
+#define VT_ATT_MIN_CHUNK 32   /* positions per attention workgroup before the cache is split further */
 #define VT_LDS_X 9216         /* staged activation vector (largest: the SwiGLU output) */
 #define VT_LDS_Y 512          /* row results of one workgroup */
 #define VT_LDS_FLOATS (VT_LDS_X + VT_LDS_Y)
