@@ -83,6 +83,28 @@ def test_predict_velocity_against_reference_fixture(ac_session):
     assert_close(gold["vel_uncond"], vu, "cfg uncond")
 
 
+def test_velocity_memo_follows_the_reference_call_pattern(ac_session):
+    """The host file asks for cond then uncond (zero hidden) velocity per Euler step
+    (voxtral_tts_acoustic.c:345-348).  The second call is answered from the batch of the
+    first; it must equal what a fresh pass gives, also for off-grid times, and a changed
+    latent or time must not be served from the memo."""
+    hip, orc, ac = ac_session
+    zeros = np.zeros(S.DIM, np.float32)
+    for t in (np.float32(2) / np.float32(7), np.float32(0.3)):
+        x = S.f32_normal(S.ACOUSTIC_DIM, 61)
+        h = S.f32_normal(S.DIM, 62)
+        vc = hip.predict_velocity(x, h, t)
+        vu = hip.predict_velocity(x, zeros, t)             # memo
+        fc, fu = hip.predict_velocity_cfg(x, h, t)         # fresh pass, both branches
+        assert np.array_equal(vc, fc) and np.array_equal(vu, fu)
+        assert_close(orc.predict_velocity(x, h, t), vc, "cond vs oracle")
+        assert_close(orc.predict_velocity(x, zeros, t), vu, "uncond vs oracle")
+        x2 = S.f32_normal(S.ACOUSTIC_DIM, 63)
+        vu2 = hip.predict_velocity(x2, zeros, t)           # other latent: computed, not remembered
+        assert_close(orc.predict_velocity(x2, zeros, t), vu2, "uncond, new latent")
+        assert not np.array_equal(vu2, vu)
+
+
 def test_acoustic_frames_codes_bit_exact(ac_session):
     """Sampled codes at a fixed seed: noise comes from the host RNG restated by
     the oracle (the reference draws it on the host too), the frame runs on the

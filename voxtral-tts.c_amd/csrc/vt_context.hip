@@ -283,7 +283,7 @@ extern "C" int tts_hip_upload_acoustic_weights(void *acoustic_ptr) {
     g_vt.ac_uploaded = 0;
     d->semantic_bias = NULL;
     d->time_tok_ready = 0;
-    if (!(d->time_tok = (float *)vt_dev_alloc(sizeof(float) * 7 * VT_DIM))) return -1;
+    if (!(d->time_tok = (float *)vt_dev_alloc(sizeof(float) * 8 * VT_DIM))) return -1;
     if (!(d->input_proj = (uint16_t *)upload(ac->input_proj_bf16, (size_t)VT_DIM * VT_AC_DIM_IN * 2))) return -1;
     if (!(d->time_proj = (uint16_t *)upload(ac->time_proj_bf16, (size_t)VT_DIM * VT_DIM * 2))) return -1;
     if (!(d->llm_proj = (uint16_t *)upload(ac->llm_proj_bf16, (size_t)VT_DIM * VT_DIM * 2))) return -1;

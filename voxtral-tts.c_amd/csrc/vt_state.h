@@ -27,7 +27,7 @@ struct vt_acoustic_dev {
     float *norm;
     float *time_inv_freq;
     float h_time_inv_freq[VT_DIM / 2];
-    float *time_tok;              /* [7, 3072] projected time tokens of the Euler grid */
+    float *time_tok;              /* [8, 3072]: projected time tokens of the Euler grid, then the last LLM token */
     int time_tok_ready;
 };
 
