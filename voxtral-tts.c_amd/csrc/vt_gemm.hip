@@ -14,10 +14,10 @@
  * Tiling: workgroup tile 128 x 128, K step 64, four waves in a 2 x 2 grid of
  * 64 x 64 wave tiles, v_mfma_f32_32x32x16_bf16.  Tiles are staged through LDS
  * with a row pitch of 144 bytes (128 of data + 16 of padding): the 16 lanes of
- * a 16-byte fragment read then cover all 64 banks once.  One LDS stage, two
- * register stages: a K step is requested two steps before it is multiplied
- * (weights come from HBM: one step of latency cover is not enough), and two
- * workgroups share a CU.  Workgroups that need the same weight tile
+ * a 16-byte fragment read then cover all 64 banks once.  One LDS stage; the
+ * next K step is fetched into registers while the current one is multiplied,
+ * the fragments of the next 16-wide slice are read while the current slice is
+ * multiplied, and two workgroups share a CU.  Workgroups that need the same weight tile
  * (the M tiles of one N tile) get consecutive slots on one XCD, so the tile is
  * fetched from HBM once and served from that XCD's L2 afterwards.  Long K can
  * be cut into `splits` ranges that write separate partial planes; the caller
@@ -75,21 +75,19 @@ vt_gemm_mfma_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const ui
         pw[i] = W + (size_t)(nt * GM_TILE + lr + 32 * i) * K + k0 + lc * 8;
     }
 
-    /* two register stages: the tile multiplied in iteration kt was requested in iteration
-     * kt - 2, so that a request has two full K steps of both resident workgroups to arrive */
-    u32x4 ra[2][4], rl[2][4], rb[2][4];
+    /* the next K step is fetched into registers while the current one is multiplied */
+    u32x4 ra[4], rl[4], rb[4];
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    auto fetch = [&](int st, int kt) {
+    auto fetch = [&](int kt) {
         const int adv = kt * GM_BK;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            ra[st][i] = live[i] ? gm_ld(pa[i] + adv) : zero;
-            rl[st][i] = live[i] ? gm_ld(pl[i] + adv) : zero;
-            rb[st][i] = gm_ld(pw[i] + adv);
+            ra[i] = live[i] ? gm_ld(pa[i] + adv) : zero;
+            rl[i] = live[i] ? gm_ld(pl[i] + adv) : zero;
+            rb[i] = gm_ld(pw[i] + adv);
         }
     };
-    fetch(0, 0);
-    if (tiles > 1) fetch(1, 1);
+    fetch(0);
 
     f32x16 acc[2][2];
 #pragma unroll
@@ -103,41 +101,50 @@ vt_gemm_mfma_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const ui
     const int fa_off = (64 * wm + (lane & 31)) * GM_ROWB + (lane >> 5) * 16;
     const int fb_off = (64 * wn + (lane & 31)) * GM_ROWB + (lane >> 5) * 16 + 2 * GM_MAT;
 
-    auto step = [&](int st, int kt) {
+    /* fragments of one 16-wide slice: hi, lo of two row blocks and the weights of two column blocks */
+    struct frags { bf16x8 fa[2], fl[2], fb[2]; };
+    auto read_frags = [&](frags &f, int ks) {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            f.fa[b] = gm_frag(lds + fa_off + 32 * b * GM_ROWB + ks * 32);
+            f.fl[b] = gm_frag(lds + GM_MAT + fa_off + 32 * b * GM_ROWB + ks * 32);
+            f.fb[b] = gm_frag(lds + fb_off + 32 * b * GM_ROWB + ks * 32);
+        }
+    };
+    auto mma = [&](const frags &f) {
+        /* four independent accumulators between two products into the same one */
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.fl[a], f.fb[b], acc[a][b], 0, 0, 0);
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+                acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.fa[a], f.fb[b], acc[a][b], 0, 0, 0);
+    };
+
+    for (int kt = 0; kt < tiles; kt++) {
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            *reinterpret_cast<u32x4 *>(lds + st_off + 32 * i * GM_ROWB) = ra[st][i];
-            *reinterpret_cast<u32x4 *>(lds + GM_MAT + st_off + 32 * i * GM_ROWB) = rl[st][i];
-            *reinterpret_cast<u32x4 *>(lds + 2 * GM_MAT + st_off + 32 * i * GM_ROWB) = rb[st][i];
+            *reinterpret_cast<u32x4 *>(lds + st_off + 32 * i * GM_ROWB) = ra[i];
+            *reinterpret_cast<u32x4 *>(lds + GM_MAT + st_off + 32 * i * GM_ROWB) = rl[i];
+            *reinterpret_cast<u32x4 *>(lds + 2 * GM_MAT + st_off + 32 * i * GM_ROWB) = rb[i];
         }
         __syncthreads();
-        if (kt + 2 < tiles) fetch(st, kt + 2);
-#pragma unroll
-        for (int ks = 0; ks < GM_BK / 16; ks++) {
-            bf16x8 fa[2], fl[2], fb[2];
-#pragma unroll
-            for (int b = 0; b < 2; b++) {
-                fa[b] = gm_frag(lds + fa_off + 32 * b * GM_ROWB + ks * 32);
-                fl[b] = gm_frag(lds + GM_MAT + fa_off + 32 * b * GM_ROWB + ks * 32);
-                fb[b] = gm_frag(lds + fb_off + 32 * b * GM_ROWB + ks * 32);
-            }
-            /* four independent accumulators between two products into the same one */
-#pragma unroll
-            for (int a = 0; a < 2; a++)
-#pragma unroll
-                for (int b = 0; b < 2; b++)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fl[a], fb[b], acc[a][b], 0, 0, 0);
-#pragma unroll
-            for (int a = 0; a < 2; a++)
-#pragma unroll
-                for (int b = 0; b < 2; b++)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fb[b], acc[a][b], 0, 0, 0);
-        }
-    };
-    for (int kt = 0; kt < tiles; kt += 2) {
-        step(0, kt);
-        if (kt + 1 < tiles) step(1, kt + 1);
+        if (kt + 1 < tiles) fetch(kt + 1);
+        /* the fragments of slice ks+1 are read while slice ks is multiplied */
+        frags f0, f1;
+        read_frags(f0, 0);
+        read_frags(f1, 1);
+        mma(f0);
+        read_frags(f0, 2);
+        mma(f1);
+        read_frags(f1, 3);
+        mma(f0);
+        mma(f1);
     }
 
     /* accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 */
