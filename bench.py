@@ -318,12 +318,88 @@ def bench_acoustic(args):
     print(json.dumps(out))
 
 
+AUDIO_ROWS = 8194 + 36 * 23
+FRAME_SECONDS = 0.08                      # one frame of codes is 80 ms of audio (12.5 Hz)
+
+
+def bench_frame(args):
+    """The whole per-frame loop of voxtral_tts.c:301-321 on the device: 26-layer backbone step,
+    acoustic frame (semantic head, 7 guided Euler steps, FSQ) and the audio-code embedding that
+    becomes the next backbone input.  A step is one frame; 64-token prompt prefilled first."""
+    import cases
+    K, W = args.steps, args.warmup
+    workers = min(16, os.cpu_count() or 8)
+    t0 = time.time()
+    layers = make_layers(N_LAYERS, workers)
+    final_norm = S.norm_weight(S.DIM, 99)
+    ac = S.Acoustic(50)
+    table = S.bf16_normal((AUDIO_ROWS, S.DIM), 4242, 0.05)
+    offs = np.zeros(S.CODES, np.int32)
+    offs[1] = 8194
+    for i in range(2, S.CODES):
+        offs[i] = offs[i - 1] + 23
+    ids = np.random.default_rng(7).integers(0, 131072, PROMPT)
+    prompt = np.stack([emb_row(t) for t in ids]).astype(np.float32)
+    t_gen = time.time() - t0
+    hip = H.Hip(kv_max=PROMPT + W + K + 8)
+    lib = hip.lib
+    t0 = time.time()
+    hip.upload_decoder(layers, final_norm, N_LAYERS)
+    hip.upload_acoustic(ac)
+    assert lib.tts_hip_upload_audio_embeddings(table.ctypes.data, AUDIO_ROWS, offs.ctypes.data) == 0
+    t_up = time.time() - t0
+    hip.llm_prefill(prompt)
+    st = C.c_uint64(0)
+    S.oracle().orc_rng_seed(C.byref(st), 42)
+    noise = np.zeros((W + K, S.ACOUSTIC_DIM), np.float32)
+    for f in range(W + K):
+        S.oracle().orc_randn_fill(C.byref(st), S.fp(noise[f]), S.ACOUSTIC_DIM)
+    d_e = H.DevBuf.from_numpy(lib, emb_row(24))          # the audio start token's stand-in
+    codes = np.zeros(S.CODES, np.int32)
+    pos = PROMPT
+    n_end = 0
+    for f in range(W):
+        lib.tts_hip_generate_frame(codes.ctypes.data, d_e.ptr, noise[f].ctypes.data, pos)
+        pos += 1
+    lib.tts_hip_sync()
+    t0 = time.time()
+    for f in range(W, W + K):
+        lib.tts_hip_generate_frame(codes.ctypes.data, d_e.ptr, noise[f].ctypes.data, pos)
+        n_end += int(codes[0] == 1)
+        pos += 1
+    lib.tts_hip_sync()
+    ms_step = (time.time() - t0) * 1e3 / K
+    hip.check()
+    fb = step_bytes(PROMPT + W + (K - 1) / 2.0) + acoustic_frame_bytes() + S.CODES * S.DIM * 2
+    out = {
+        "metric": "generation loop ms/frame (backbone step + acoustic frame + code embedding)",
+        "value": round(ms_step, 4), "unit": "ms/frame",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 activations, bf16 weights", "data": "synthetic",
+        "config": {"workload": "per-frame generation loop on the device (configs[2] + configs[4] chained through the "
+                               "audio-code embedding), 64-token prompt", "layers": N_LAYERS,
+                   "timed": "host clock over whole frames; per frame 36 floats of noise go in, 37 codes come back"},
+        "frames_per_s": round(1000.0 / ms_step, 1),
+        "realtime_factor": round(FRAME_SECONDS * 1000.0 / ms_step, 1),
+        "end_audio_frames": n_end,
+        "roofline": {"kernel": "whole frame (vt_decode_step_kernel + 84 vt_ac_phase_kernel launches)", "bound": "hbm",
+                     "achieved": round(fb / (ms_step * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(fb / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_frame": int(fb)},
+        "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
+        "cpu_baseline": None,
+    }
+    hip.close()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=("decode", "prefill", "acoustic"), default="decode",
+    ap.add_argument("--workload", choices=("decode", "prefill", "acoustic", "frame"), default="decode",
                     help="decode = the headline metric; prefill / acoustic = the other two configurations")
     ap.add_argument("--mode", type=int, default=0, help="0 persistent kernel, 1 per-phase kernels, 2 streaming kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
@@ -341,6 +417,8 @@ def main():
         return bench_prefill(args)
     if args.workload == "acoustic":
         return bench_acoustic(args)
+    if args.workload == "frame":
+        return bench_frame(args)
     K, W = args.steps, args.warmup
     workers = min(16, os.cpu_count() or 8)
 

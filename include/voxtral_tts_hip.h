@@ -192,6 +192,19 @@ void tts_hip_predict_velocity_cfg(float *out_v_cond, float *out_v_uncond, const 
 void tts_hip_acoustic_frame(int *out_codes, const float *llm_hidden, const float *x0,
                             float *out_x);
 
+/* Audio-code embedding table bf16 [total_rows, 3072] and the first row of each of the 37
+ * codebooks (tts_audio_embed_t, voxtral_tts.h:226-236; tts_audio_embed_load,
+ * voxtral_tts_voice.c:251-290).  Host or device pointers; copies.  0 / -1. */
+int tts_hip_upload_audio_embeddings(const uint16_t *emb_bf16, int total_rows, const int *offsets);
+/* replaces tts_audio_embed_forward (voxtral_tts_voice.c:292-315): host codes [37] -> host
+ * embedding [3072], the 37 rows summed in codebook order; synchronous. */
+void tts_hip_audio_embed(float *out_embed, const int *codes);
+/* One turn of the generation loop of voxtral_tts.c:301-321 on the device: backbone step at
+ * cache position pos on d_embed (device, f32 [3072]) -> frame of 37 codes from the noise x0
+ * (host, f32 [36]) -> embedding of the codes written back to d_embed.  Synchronous; returns
+ * the codes (END_AUDIO: codes[0] == 1, the rest 2). */
+void tts_hip_generate_frame(int *out_codes, float *d_embed, const float *x0, int pos);
+
 /* Decode schedule: 0 = persistent whole-step kernel (default), 1 = one kernel per
  * phase, 2 = streaming whole-step kernel (256-CU devices; experimental). */
 void tts_hip_set_decode_mode(int mode);

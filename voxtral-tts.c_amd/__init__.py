@@ -96,6 +96,9 @@ SIGNATURES = {
     "tts_hip_timer_start": (None, []),
     "tts_hip_timer_stop_ms": (C.c_float, []),
     "tts_hip_bench_kernel": (C.c_float, [C.c_int, C.c_int]),
+    "tts_hip_upload_audio_embeddings": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
+    "tts_hip_audio_embed": (None, [C.c_void_p, C.c_void_p]),
+    "tts_hip_generate_frame": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]),
 }
 
 _lib = None

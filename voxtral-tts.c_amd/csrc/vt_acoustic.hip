@@ -680,37 +680,118 @@ extern "C" void tts_hip_predict_velocity_cfg(float *out_v_cond, float *out_v_unc
     predict(out_v_cond, out_v_uncond, x_t, llm_hidden, t_val);
 }
 
-extern "C" void tts_hip_acoustic_frame(int *out_codes, const float *llm_hidden, const float *x0,
-                                       float *out_x) {
-    if (!ac_ready("tts_hip_acoustic_frame")) return;
+/* Enqueues one frame: semantic head + argmax, 7 guided Euler steps, FSQ.  d_or_h_hidden may
+ * be a host or a device pointer.  Codes end up in w->codes, the latent in w->x; nothing is
+ * synchronised. */
+static int enqueue_frame(ac_work *w, const float *d_or_h_hidden, const float *x0) {
     hipStream_t st = g_vt.stream;
     vt_acoustic_dev *ac = &g_vt.ac;
     float *base = (float *)vt_scratch(sizeof(float) * AC_WORK_FLOATS);
-    if (!base) return;
-    ac_work w;
-    carve(&w, base);
+    if (!base) return -1;
+    carve(w, base);
     float ts[AC_STEPS + 1];
     for (int i = 0; i <= AC_STEPS; i++) ts[i] = (float)i / (float)AC_STEPS;
-    if (ensure_time_grid(w.temb)) return;                /* the projected time tokens depend on the weights only */
-    VT_TRYV(hipMemcpyAsync(w.hidden, llm_hidden, sizeof(float) * VT_DIM, hipMemcpyDefault, st));
-    VT_TRYV(hipMemcpyAsync(w.x, x0, sizeof(float) * VT_AC_DIM_IN, hipMemcpyDefault, st));
-    vt_launch_linear(w.logits, w.hidden, ac->semantic_out, ac->semantic_bias, 1, VT_DIM, VT_SEM_PADDED);
-    hipLaunchKernelGGL(vt_semantic_argmax_kernel, dim3(1), dim3(1024), 0, st, w.logits, w.codes);
-    vt_launch_linear(w.llm_tok, w.hidden, ac->llm_proj, NULL, 1, VT_DIM, VT_DIM);
+    if (ensure_time_grid(w->temb)) return -1;            /* the projected time tokens depend on the weights only */
+    if (vt_check(hipMemcpyAsync(w->hidden, d_or_h_hidden, sizeof(float) * VT_DIM, hipMemcpyDefault, st), "frame hidden")) return -1;
+    if (vt_check(hipMemcpyAsync(w->x, x0, sizeof(float) * VT_AC_DIM_IN, hipMemcpyDefault, st), "frame noise")) return -1;
+    vt_launch_linear(w->logits, w->hidden, ac->semantic_out, ac->semantic_bias, 1, VT_DIM, VT_SEM_PADDED);
+    hipLaunchKernelGGL(vt_semantic_argmax_kernel, dim3(1), dim3(1024), 0, st, w->logits, w->codes);
+    vt_launch_linear(w->llm_tok, w->hidden, ac->llm_proj, NULL, 1, VT_DIM, VT_DIM);
     /* the flow runs without waiting for the semantic code; an END_AUDIO frame discards it */
-    launch_edge(&w, ac->time_tok, w.llm_tok, 0.f, 0, 0, 1, 0);
+    launch_edge(w, ac->time_tok, w->llm_tok, 0.f, 0, 0, 1, 0);
     for (int s = 0; s < AC_STEPS; s++) {
         volatile float dt = ts[s + 1] - ts[s];
-        if (run_layers(&w)) return;
+        if (run_layers(w)) return -1;
         const int last = s + 1 == AC_STEPS;
-        launch_edge(&w, ac->time_tok + (size_t)(last ? s : s + 1) * VT_DIM, w.llm_tok, (float)dt, 1, 1, !last, last);
+        launch_edge(w, ac->time_tok + (size_t)(last ? s : s + 1) * VT_DIM, w->llm_tok, (float)dt, 1, 1, !last, last);
     }
-    VT_TRYV(hipGetLastError());
-    VT_TRYV(hipStreamSynchronize(st));
-    VT_TRYV(hipMemcpy(out_codes, w.codes, sizeof(int) * (1 + VT_AC_DIM_IN), hipMemcpyDeviceToHost));
-    if (out_x) VT_TRYV(hipMemcpy(out_x, w.x, sizeof(float) * VT_AC_DIM_IN, hipMemcpyDeviceToHost));
+    return vt_check(hipGetLastError(), "frame launch");
+}
+
+static void finish_frame(const ac_work *w, int *out_codes, float *out_x) {
+    VT_TRYV(hipStreamSynchronize(g_vt.stream));
+    VT_TRYV(hipMemcpy(out_codes, w->codes, sizeof(int) * (1 + VT_AC_DIM_IN), hipMemcpyDeviceToHost));
+    if (out_x) VT_TRYV(hipMemcpy(out_x, w->x, sizeof(float) * VT_AC_DIM_IN, hipMemcpyDeviceToHost));
     if (out_codes[0] == 1) {                            /* END_AUDIO */
         for (int i = 1; i <= VT_AC_DIM_IN; i++) out_codes[i] = 2;
         if (out_x) memset(out_x, 0, sizeof(float) * VT_AC_DIM_IN);
     }
+}
+
+extern "C" void tts_hip_acoustic_frame(int *out_codes, const float *llm_hidden, const float *x0,
+                                       float *out_x) {
+    if (!ac_ready("tts_hip_acoustic_frame")) return;
+    ac_work w;
+    if (enqueue_frame(&w, llm_hidden, x0)) return;
+    finish_frame(&w, out_codes, out_x);
+}
+
+/* ---- audio-code embedding and the per-frame loop -------------------------------------- */
+
+/* out[i] = sum over the 37 codebooks, in codebook order, of row offsets[cb] + codes[cb] of the
+ * bf16 table, starting from 0 (tts_audio_embed_forward, voxtral_tts_voice.c:292-315): the same
+ * fp32 additions in the same order, so the result is bit-equal to the CPU's. */
+__global__ void vt_audio_embed_kernel(float *out, const uint16_t *emb, const int *offsets, const int *codes,
+                                      int total_rows) {
+    const int i = (int)(blockIdx.x * blockDim.x + threadIdx.x);
+    if (i >= VT_DIM) return;
+    float acc = 0.0f;
+    for (int cb = 0; cb < 1 + VT_AC_DIM_IN; cb++) {
+        int row = offsets[cb] + codes[cb];
+        row = row < 0 ? 0 : (row >= total_rows ? total_rows - 1 : row);
+        acc = __fadd_rn(acc, __uint_as_float((unsigned)emb[(size_t)row * VT_DIM + i] << 16));
+    }
+    out[i] = acc;
+}
+
+extern "C" int tts_hip_upload_audio_embeddings(const uint16_t *emb_bf16, int total_rows, const int *offsets) {
+    if (!g_vt.initialized) { vt_set_error("tts_hip_upload_audio_embeddings: backend not initialised"); return -1; }
+    if (!emb_bf16 || !offsets || total_rows < 1) { vt_set_error("tts_hip_upload_audio_embeddings: bad arguments"); return -1; }
+    vt_acoustic_dev *ac = &g_vt.ac;
+    if (ac->audio_emb) (void)hipFree(ac->audio_emb);
+    if (ac->audio_offsets) (void)hipFree(ac->audio_offsets);
+    ac->audio_rows = 0;
+    const size_t bytes = (size_t)total_rows * VT_DIM * 2;
+    if (!(ac->audio_emb = (uint16_t *)vt_dev_alloc(bytes))) return -1;
+    if (!(ac->audio_offsets = (int *)vt_dev_alloc(sizeof(int) * 2 * (1 + VT_AC_DIM_IN)))) return -1;
+    VT_TRY(hipMemcpy(ac->audio_emb, emb_bf16, bytes, hipMemcpyDefault));
+    VT_TRY(hipMemcpy(ac->audio_offsets, offsets, sizeof(int) * (1 + VT_AC_DIM_IN), hipMemcpyDefault));
+    ac->audio_rows = total_rows;
+    return 0;
+}
+
+static int embed_ready(const char *who) {
+    if (g_vt.initialized && g_vt.ac.audio_rows > 0) return 1;
+    vt_set_error("%s: audio embeddings not uploaded", who);
+    return 0;
+}
+
+/* host codes [37] -> host embedding [3072]; synchronous */
+extern "C" void tts_hip_audio_embed(float *out_embed, const int *codes) {
+    if (!embed_ready("tts_hip_audio_embed")) return;
+    vt_acoustic_dev *ac = &g_vt.ac;
+    hipStream_t st = g_vt.stream;
+    int *d_codes = ac->audio_offsets + (1 + VT_AC_DIM_IN);
+    VT_TRYV(hipStreamSynchronize(st));
+    VT_TRYV(hipMemcpy(d_codes, codes, sizeof(int) * (1 + VT_AC_DIM_IN), hipMemcpyHostToDevice));
+    hipLaunchKernelGGL(vt_audio_embed_kernel, dim3(VT_DIM / 256), dim3(256), 0, st, g_vt.d_embed, ac->audio_emb,
+                       ac->audio_offsets, d_codes, ac->audio_rows);
+    VT_TRYV(hipStreamSynchronize(st));
+    VT_TRYV(hipMemcpy(out_embed, g_vt.d_embed, sizeof(float) * VT_DIM, hipMemcpyDeviceToHost));
+}
+
+/* One turn of the generation loop (voxtral_tts.c:301-321) without leaving the device in
+ * between: backbone step at cache position pos on d_embed -> hidden -> frame of 37 codes ->
+ * embedding of those codes back into d_embed.  x0 is the frame's noise (host, 36 floats: the
+ * caller keeps the RNG).  Returns the codes; after an END_AUDIO frame d_embed is not meaningful. */
+extern "C" void tts_hip_generate_frame(int *out_codes, float *d_embed, const float *x0, int pos) {
+    if (!ac_ready("tts_hip_generate_frame") || !embed_ready("tts_hip_generate_frame")) return;
+    if (g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_generate_frame: no backbone weights uploaded"); return; }
+    if (vt_run_step(g_vt.d_layers, g_vt.n_dec_layers, 0, g_vt.d_dec_norm, d_embed, g_vt.d_hidden, pos)) return;
+    ac_work w;
+    if (enqueue_frame(&w, g_vt.d_hidden, x0)) return;
+    vt_acoustic_dev *ac = &g_vt.ac;
+    hipLaunchKernelGGL(vt_audio_embed_kernel, dim3(VT_DIM / 256), dim3(256), 0, g_vt.stream, d_embed, ac->audio_emb,
+                       ac->audio_offsets, w.codes, ac->audio_rows);
+    finish_frame(&w, out_codes, NULL);
 }

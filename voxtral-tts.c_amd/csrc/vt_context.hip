@@ -158,7 +158,8 @@ extern "C" void tts_hip_free(void) {
     void *ptrs[] = {g_vt.d_layers, g_vt.d_dec_norm, g_vt.d_tok_emb, g_vt.ac.input_proj,
                     g_vt.ac.time_proj, g_vt.ac.llm_proj, g_vt.ac.semantic_out,
                     g_vt.ac.acoustic_out, g_vt.ac.semantic_bias, g_vt.ac.norm,
-                    g_vt.ac.time_inv_freq, g_vt.ac.time_tok, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu,
+                    g_vt.ac.time_inv_freq, g_vt.ac.time_tok, g_vt.ac.audio_emb, g_vt.ac.audio_offsets,
+                    g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu,
                     g_vt.d_rope, g_vt.d_x, g_vt.d_q, g_vt.d_attn, g_vt.d_h, g_vt.d_att_part,
                     g_vt.d_att_cnt, g_vt.d_embed, g_vt.d_hidden, g_vt.d_bar_flags,
                     g_vt.d_abort, g_vt.d_dummy, g_vt.d_scratch};

@@ -29,6 +29,9 @@ struct vt_acoustic_dev {
     float h_time_inv_freq[VT_DIM / 2];
     float *time_tok;              /* [8, 3072]: projected time tokens of the Euler grid, then the last LLM token */
     int time_tok_ready;
+    uint16_t *audio_emb;          /* [audio_rows, 3072] audio-code embedding table */
+    int *audio_offsets;           /* [37] first row of every codebook, then 37 ints of staging for codes */
+    int audio_rows;
 };
 
 struct vt_state {
