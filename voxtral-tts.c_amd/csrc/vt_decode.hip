@@ -65,17 +65,20 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
     vt_qkv_prefetch(ring, a.layers[0]);
     for (int l = 0; l < a.n_layers; l++) {
         const vt_layer_dev L = a.layers[l];
-        vt_qkv_body(ring, L, a, l, x_in, lds);
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_wo_prefetch(ring, L); }, tn)) return;
+        /* the next phase's first row is requested as soon as the ring is free, the other rows
+         * between arriving at the barrier and waiting on it: together they keep the HBM pipe
+         * busy from the end of one phase's arithmetic to the start of the next one's */
+        const bool more = l + 1 < a.n_layers;
+        vt_qkv_body(ring, L, a, l, x_in, lds, [&] { vt_wo_prefetch(ring, L, VT_PART_HEAD); });
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_wo_prefetch(ring, L, VT_PART_TAIL); }, tn)) return;
         vt_attn_phase(a, l, lds);
         if (!vt_barrier_then(gs, &s_flag, [] {}, tn)) return;
-        vt_wo_body(ring, L, a, x_in, lds);
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L); }, tn)) return;
-        vt_w13_body(ring, L, a, lds);
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w2_prefetch(ring, L); }, tn)) return;
-        vt_w2_body(ring, L, a, lds);
-        const bool more = l + 1 < a.n_layers;
-        if (!vt_barrier_then(gs, &s_flag, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1]); }, tn))
+        vt_wo_body(ring, L, a, x_in, lds, [&] { vt_w13_prefetch(ring, L, VT_PART_HEAD); });
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L, VT_PART_TAIL); }, tn)) return;
+        vt_w13_body(ring, L, a, lds, [&] { vt_w2_prefetch(ring, L, VT_PART_HEAD); });
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w2_prefetch(ring, L, VT_PART_TAIL); }, tn)) return;
+        vt_w2_body(ring, L, a, lds, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1], VT_PART_HEAD); });
+        if (!vt_barrier_then(gs, &s_flag, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1], VT_PART_TAIL); }, tn))
             return;
         x_in = a.x;
     }

@@ -166,15 +166,20 @@ __device__ __forceinline__ vt_rows vt_split_rows(int n_rows, int align, int k_pe
     return r;
 }
 
-/* Request the first D rows of a wave's share. */
+/* Request rows j0 .. j1-1 of the first D rows of a wave's share.  The persistent kernel asks
+ * for the first row as soon as the previous phase has multiplied its ring out (PART_HEAD),
+ * and for the others after it has handed its results over (PART_TAIL). */
+enum { VT_PART_ALL = 0, VT_PART_HEAD = 1, VT_PART_TAIL = 2 };
+
 template <int NK, int D>
 __device__ __forceinline__ void vt_ring_prefetch(u32x4 (&ring)[VT_RING], const uint16_t *W,
-                                                 int row_len, const vt_rows &r) {
+                                                 int row_len, const vt_rows &r, int part = VT_PART_ALL) {
     static_assert(NK * D <= VT_RING, "ring too small");
     const uint16_t *base = W + (size_t)r.r0 * row_len + r.kofs + vt_lane() * 8;
+    const int j0 = part == VT_PART_TAIL ? 1 : 0, j1 = part == VT_PART_HEAD ? 1 : D;
 #pragma unroll
     for (int j = 0; j < D; j++) {
-        if (j < r.nr) {
+        if (j >= j0 && j < j1 && j < r.nr) {
 #pragma unroll
             for (int c = 0; c < NK; c++)
                 ring[j * NK + c] = vt_ldw(base + (size_t)j * row_len + c * 512);
@@ -217,19 +222,26 @@ __device__ __forceinline__ void vt_ring_run(u32x4 (&ring)[VT_RING], const uint16
 
 __device__ __forceinline__ vt_rows vt_qkv_rows() { return vt_split_rows<1>(VT_QKV_DIM, 2, 0); }
 
-__device__ __forceinline__ void vt_qkv_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L) {
-    vt_ring_prefetch<6, 3>(ring, L.wqkv, VT_DIM, vt_qkv_rows());
+__device__ __forceinline__ void vt_qkv_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
+                                                int part = VT_PART_ALL) {
+    vt_ring_prefetch<6, 3>(ring, L.wqkv, VT_DIM, vt_qkv_rows(), part);
 }
 
+struct vt_nothing { __device__ __forceinline__ void operator()() const {} };
+
+/* `after_run` is called when the ring has been multiplied out and is free again, before the
+ * results are stored. */
+template <class AR = vt_nothing>
 __device__ __forceinline__ void vt_qkv_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
                                             const vt_step_args &a, int layer,
-                                            const float *x_in, float *lds) {
+                                            const float *x_in, float *lds, AR after_run = AR()) {
     const vt_rows r = vt_qkv_rows();
     float *lds_y = lds + VT_LDS_X;
     vt_stage(lds, x_in, VT_DIM);
     f32x4 xa[6], xb[6];
     vt_rmsnorm_slice(xa, xb, lds, L.attn_norm);
     vt_ring_run<6, 3>(ring, L.wqkv, VT_DIM, r, xa, xb, lds_y);
+    after_run();
     __syncthreads();
     /* RoPE on adjacent pairs (voxtral_tts_kernels.c:616-634), then q to its
      * buffer and k, v straight into row `pos` of the cache. */
@@ -397,22 +409,29 @@ __device__ __forceinline__ void vt_attn_phase(const vt_step_args &a, int layer, 
 
 __device__ __forceinline__ vt_rows vt_wo_rows() { return vt_split_rows<2>(VT_DIM, 1, VT_Q_DIM / 2); }
 
-__device__ __forceinline__ void vt_wo_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L) {
-    vt_ring_prefetch<4, 4>(ring, L.wo, VT_Q_DIM, vt_wo_rows());
+__device__ __forceinline__ void vt_wo_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
+                                               int part = VT_PART_ALL) {
+    vt_ring_prefetch<4, 4>(ring, L.wo, VT_Q_DIM, vt_wo_rows(), part);
 }
 
+template <class AR = vt_nothing>
 __device__ __forceinline__ void vt_wo_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
-                                           const vt_step_args &a, const float *x_in, float *lds) {
+                                           const vt_step_args &a, const float *x_in, float *lds,
+                                           AR after_run = AR()) {
     const vt_rows r = vt_wo_rows();
     float *lds_y = lds + VT_LDS_X;
     vt_stage(lds, a.attn, VT_Q_DIM);
     f32x4 xa[4], xb[4];
     vt_slice_lds<4>(xa, xb, lds, r.kofs);
+    /* the residual value of this thread's row, requested before any bulk load of the next phase */
+    const int tr = (int)threadIdx.x < r.wg_nrows ? (int)threadIdx.x : 0;
+    const float prev = vt_ldc(x_in + r.wg_row0 + tr);
     vt_ring_run<4, 4>(ring, L.wo, VT_Q_DIM, r, xa, xb, lds_y);
+    after_run();
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows; t += (int)blockDim.x) {
         const float y = lds_y[t] + lds_y[r.wg_nrows + t];
-        vt_stc(a.x + r.wg_row0 + t, vt_ldc(x_in + r.wg_row0 + t) + y);
+        vt_stc(a.x + r.wg_row0 + t, (t == tr ? prev : vt_ldc(x_in + r.wg_row0 + t)) + y);
     }
 }
 
@@ -420,18 +439,21 @@ __device__ __forceinline__ void vt_wo_body(u32x4 (&ring)[VT_RING], const vt_laye
 
 __device__ __forceinline__ vt_rows vt_w13_rows() { return vt_split_rows<1>(2 * VT_FFN, 2, 0); }
 
-__device__ __forceinline__ void vt_w13_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L) {
-    vt_ring_prefetch<6, 3>(ring, L.w13, VT_DIM, vt_w13_rows());
+__device__ __forceinline__ void vt_w13_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
+                                                int part = VT_PART_ALL) {
+    vt_ring_prefetch<6, 3>(ring, L.w13, VT_DIM, vt_w13_rows(), part);
 }
 
+template <class AR = vt_nothing>
 __device__ __forceinline__ void vt_w13_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
-                                            const vt_step_args &a, float *lds) {
+                                            const vt_step_args &a, float *lds, AR after_run = AR()) {
     const vt_rows r = vt_w13_rows();
     float *lds_y = lds + VT_LDS_X;
     vt_stage(lds, a.x, VT_DIM);
     f32x4 xa[6], xb[6];
     vt_rmsnorm_slice(xa, xb, lds, L.ffn_norm);
     vt_ring_run<6, 3>(ring, L.w13, VT_DIM, r, xa, xb, lds_y);
+    after_run();
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows / 2; t += (int)blockDim.x) {
         const float g = lds_y[2 * t], u = lds_y[2 * t + 1];
@@ -444,22 +466,27 @@ __device__ __forceinline__ void vt_w13_body(u32x4 (&ring)[VT_RING], const vt_lay
 
 __device__ __forceinline__ vt_rows vt_w2_rows() { return vt_split_rows<2>(VT_DIM, 1, VT_FFN / 2); }
 
-__device__ __forceinline__ void vt_w2_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L) {
-    vt_ring_prefetch<9, 2>(ring, L.w2, VT_FFN, vt_w2_rows());
+__device__ __forceinline__ void vt_w2_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
+                                               int part = VT_PART_ALL) {
+    vt_ring_prefetch<9, 2>(ring, L.w2, VT_FFN, vt_w2_rows(), part);
 }
 
+template <class AR = vt_nothing>
 __device__ __forceinline__ void vt_w2_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
-                                           const vt_step_args &a, float *lds) {
+                                           const vt_step_args &a, float *lds, AR after_run = AR()) {
     const vt_rows r = vt_w2_rows();
     float *lds_y = lds + VT_LDS_X;
     vt_stage(lds, a.h, VT_FFN);
     f32x4 xa[9], xb[9];
     vt_slice_lds<9>(xa, xb, lds, r.kofs);
+    const int tr = (int)threadIdx.x < r.wg_nrows ? (int)threadIdx.x : 0;
+    const float prev = vt_ldc(a.x + r.wg_row0 + tr);
     vt_ring_run<9, 2>(ring, L.w2, VT_FFN, r, xa, xb, lds_y);
+    after_run();
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows; t += (int)blockDim.x) {
         const float y = lds_y[t] + lds_y[r.wg_nrows + t];
-        vt_stc(a.x + r.wg_row0 + t, vt_ldc(a.x + r.wg_row0 + t) + y);
+        vt_stc(a.x + r.wg_row0 + t, (t == tr ? prev : vt_ldc(a.x + r.wg_row0 + t)) + y);
     }
 }
 
