@@ -166,23 +166,28 @@ __device__ __forceinline__ vt_rows vt_split_rows(int n_rows, int align, int k_pe
     return r;
 }
 
-/* Request rows j0 .. j1-1 of the first D rows of a wave's share.  The persistent kernel asks
- * for the first row as soon as the previous phase has multiplied its ring out (PART_HEAD),
- * and for the others after it has handed its results over (PART_TAIL). */
+/* Request the first D rows of a wave's share.  The persistent kernel asks for the first
+ * VT_HEAD_SLOTS slots as soon as the previous phase has multiplied its ring out (PART_HEAD)
+ * and for the others after it has handed its results over (PART_TAIL): 6 KB per wave is
+ * 48 KB per CU, about what a CU accepts as outstanding loads; more would hold up the
+ * acknowledgement of the hand-over stores that the barrier waits for. */
 enum { VT_PART_ALL = 0, VT_PART_HEAD = 1, VT_PART_TAIL = 2 };
+#define VT_HEAD_SLOTS 6        /* ring slots (KB per wave) requested ahead of the hand-over */
 
 template <int NK, int D>
 __device__ __forceinline__ void vt_ring_prefetch(u32x4 (&ring)[VT_RING], const uint16_t *W,
                                                  int row_len, const vt_rows &r, int part = VT_PART_ALL) {
     static_assert(NK * D <= VT_RING, "ring too small");
     const uint16_t *base = W + (size_t)r.r0 * row_len + r.kofs + vt_lane() * 8;
-    const int j0 = part == VT_PART_TAIL ? 1 : 0, j1 = part == VT_PART_HEAD ? 1 : D;
 #pragma unroll
     for (int j = 0; j < D; j++) {
-        if (j >= j0 && j < j1 && j < r.nr) {
+        if (j < r.nr) {
 #pragma unroll
-            for (int c = 0; c < NK; c++)
-                ring[j * NK + c] = vt_ldw(base + (size_t)j * row_len + c * 512);
+            for (int c = 0; c < NK; c++) {
+                const bool head = j * NK + c < VT_HEAD_SLOTS;
+                if (part == VT_PART_ALL || (part == VT_PART_HEAD) == head)
+                    ring[j * NK + c] = vt_ldw(base + (size_t)j * row_len + c * 512);
+            }
         }
     }
 }
