@@ -205,6 +205,22 @@ void tts_hip_audio_embed(float *out_embed, const int *codes);
  * the codes (END_AUDIO: codes[0] == 1, the rest 2). */
 void tts_hip_generate_frame(int *out_codes, float *d_embed, const float *x0, int pos);
 
+/* Checkpoint file -> device in one call, in place of the host-side loading that precedes
+ * the uploads in the reference (safetensors_open / safetensors_find / safetensors_data,
+ * voxtral_tts_safetensors.c:204-405; tts_decoder_load, voxtral_tts_llm.c:45-100;
+ * tts_acoustic_load, voxtral_tts_acoustic.c:40-130; tts_audio_embed_load,
+ * voxtral_tts_voice.c:251-290).  Maps the .safetensors file and uploads what it holds under
+ * the reference's tensor names: backbone layers 0..n-1 (as many consecutive ones as are
+ * present) with norm.weight and the token embeddings, the acoustic transformer, the
+ * audio-code embedding table.  Returns a bit mask (1 backbone, 2 acoustic, 4 audio-code
+ * embeddings) or -1; tts_hip_init first. */
+int tts_hip_load_safetensors(const char *path);
+/* Looks one tensor of a .safetensors file up without touching the GPU (safetensors_find,
+ * voxtral_tts_safetensors.c:330-345): 0 and dtype (8 chars), rank, shape (4 entries) and
+ * byte size; 1 if the file has no such tensor; -1 if the file cannot be read. */
+int tts_hip_safetensors_probe(const char *path, const char *name, char *dtype8, int *rank,
+                              long long *shape4, long long *nbytes);
+
 /* Decode schedule: 0 = persistent whole-step kernel (default), 1 = one kernel per
  * phase, 2 = streaming whole-step kernel (256-CU devices; experimental). */
 void tts_hip_set_decode_mode(int mode);

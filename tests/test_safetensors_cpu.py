@@ -1,0 +1,108 @@
+"""Header reader of the checkpoint loader (host code, no GPU): files written by the
+`safetensors` package itself are the known answers, so the reader is checked against the
+format's own writer rather than against a writer of ours (reference reader:
+voxtral_tts_safetensors.c:17-300)."""
+import ctypes as C
+import json
+import struct
+
+import numpy as np
+import pytest
+import torch
+from safetensors.torch import save_file
+
+import hipsupport as H
+
+
+def probe(lib, path, name):
+    dtype = C.create_string_buffer(8)
+    rank = C.c_int(-1)
+    shape = (C.c_longlong * 4)()
+    nbytes = C.c_longlong(-1)
+    rc = lib.tts_hip_safetensors_probe(str(path).encode(), name.encode(), dtype, C.byref(rank),
+                                       shape, C.byref(nbytes))
+    return rc, dtype.value.decode(), rank.value, list(shape), nbytes.value
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return H.load_package().lib()
+
+
+def test_probe_reads_what_the_format_writer_wrote(lib, tmp_path):
+    tensors = {
+        "layers.0.attention.wq.weight": torch.zeros(8, 6, dtype=torch.bfloat16),
+        "norm.weight": torch.arange(5, dtype=torch.float32),
+        "acoustic_transformer.layers.2.ffn_norm.weight": torch.ones(3, dtype=torch.float16),
+        "a.scalar": torch.tensor(3.0),
+        "cube": torch.zeros(2, 3, 4, 5, dtype=torch.bfloat16),
+    }
+    path = tmp_path / "m.safetensors"
+    save_file(tensors, str(path), metadata={"format": "pt", "note": "braces } ] \" in a string"})
+    want = {"layers.0.attention.wq.weight": ("BF16", [8, 6], 96),
+            "norm.weight": ("F32", [5], 20),
+            "acoustic_transformer.layers.2.ffn_norm.weight": ("F16", [3], 6),
+            "a.scalar": ("F32", [], 4),
+            "cube": ("BF16", [2, 3, 4, 5], 240)}
+    for name, (dt, shp, nb) in want.items():
+        rc, dtype, rank, shape, nbytes = probe(lib, path, name)
+        assert rc == 0, name
+        assert (dtype, rank, shape[:rank], nbytes) == (dt, len(shp), shp, nb), name
+    assert probe(lib, path, "layers.0.attention.wq")[0] == 1         # prefix of a name: absent
+    assert probe(lib, path, "__metadata__")[0] == 1                  # not a tensor
+
+
+def test_many_tensors_grow_the_index(lib, tmp_path):
+    tensors = {f"t.{i}": torch.full((i % 7 + 1,), float(i)) for i in range(1300)}
+    path = tmp_path / "many.safetensors"
+    save_file(tensors, str(path))
+    for i in (0, 511, 512, 1299):
+        rc, dtype, rank, shape, nbytes = probe(lib, path, f"t.{i}")
+        assert (rc, dtype, rank, shape[0], nbytes) == (0, "F32", 1, i % 7 + 1, 4 * (i % 7 + 1))
+
+
+def raw_file(path, header, data=b""):
+    h = header if isinstance(header, bytes) else json.dumps(header).encode()
+    path.write_bytes(struct.pack("<Q", len(h)) + h + data)
+
+
+def test_malformed_files_are_errors(lib, tmp_path):
+    n0 = lib.tts_hip_error_count()
+    assert probe(lib, tmp_path / "absent.safetensors", "x")[0] == -1
+    p = tmp_path / "short.safetensors"
+    p.write_bytes(b"\x01\x02")
+    assert probe(lib, p, "x")[0] == -1
+    # header length beyond the file
+    p = tmp_path / "len.safetensors"
+    p.write_bytes(struct.pack("<Q", 1 << 40) + b"{}")
+    assert probe(lib, p, "x")[0] == -1
+    # tensor bytes beyond the data section
+    p = tmp_path / "range.safetensors"
+    raw_file(p, {"x": {"dtype": "F32", "shape": [4], "data_offsets": [0, 16]}}, b"\0" * 8)
+    assert probe(lib, p, "x")[0] == -1
+    # cut-off JSON
+    p = tmp_path / "cut.safetensors"
+    raw_file(p, b'{"x":{"dtype":"F32","shape":[4],"data_offsets":[0,')
+    assert probe(lib, p, "x")[0] == -1
+    # an entry without offsets
+    p = tmp_path / "nooff.safetensors"
+    raw_file(p, {"x": {"dtype": "F32", "shape": [4]}}, b"\0" * 16)
+    assert probe(lib, p, "x")[0] == -1
+    assert lib.tts_hip_error_count() == n0 + 6
+    # and a well-formed hand-written one, keys in another order, unknown keys skipped
+    p = tmp_path / "ok.safetensors"
+    raw_file(p, b' { "x" : { "data_offsets" : [ 0 , 16 ] , "extra" : {"a":[1,{"b":null}]} ,'
+                b' "shape" : [ 2 , 2 ] , "dtype" : "F32" } } ', b"\0" * 16)
+    assert probe(lib, p, "x")[:3] == (0, "F32", 2)
+    p = tmp_path / "empty.safetensors"
+    raw_file(p, b"{}")
+    assert probe(lib, p, "x")[0] == 1
+
+
+def test_load_needs_an_initialised_backend(lib, tmp_path):
+    n0 = lib.tts_hip_error_count()
+    p = tmp_path / "e.safetensors"
+    raw_file(p, b"{}")
+    if not H.load_package().ctx().initialized:
+        assert lib.tts_hip_load_safetensors(str(p).encode()) == -1
+        assert lib.tts_hip_error_count() == n0 + 1

@@ -99,6 +99,9 @@ SIGNATURES = {
     "tts_hip_upload_audio_embeddings": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "tts_hip_audio_embed": (None, [C.c_void_p, C.c_void_p]),
     "tts_hip_generate_frame": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]),
+    "tts_hip_load_safetensors": (C.c_int, [C.c_char_p]),
+    "tts_hip_safetensors_probe": (C.c_int, [C.c_char_p, C.c_char_p, C.c_char_p, C.c_void_p,
+                                            C.c_void_p, C.c_void_p]),
 }
 
 _lib = None
