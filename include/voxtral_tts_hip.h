@@ -66,6 +66,34 @@ typedef struct {
     tts_hip_host_layer_t layers[TTS_HIP_AC_LAYERS];
 } tts_hip_host_acoustic_t;
 
+/* Audio codec decoder weights: field order and types equal tts_conv_t / tts_codec_layer_t /
+ * tts_codec_t (voxtral_tts.h:172-225), so a pointer to the reference's struct can be passed
+ * unchanged.  All tensors fp32 (weight norm already folded, voxtral_tts_codec.c:38-57). */
+typedef struct {
+    float *weight;            /* conv1d [out_ch, in_ch, kernel]; transposed [in_ch, out_ch, kernel] */
+    float *bias;              /* [out_ch] or NULL */
+    int in_ch, out_ch, kernel, stride, is_transpose;
+} tts_hip_host_conv_t;
+
+typedef struct {
+    float *wq, *wk, *wv, *wo; /* [1024, 1024] */
+    float *q_norm, *k_norm;   /* [1024] or NULL */
+    float *attention_norm;    /* [1024] */
+    float *w1, *w2, *w3;      /* [4096, 1024] [1024, 4096] [4096, 1024] */
+    float *ffn_norm;          /* [1024] */
+    float *attn_scale, *ffn_scale;   /* [1024] layer scale, or NULL */
+    int window_size;
+} tts_hip_host_codec_layer_t;
+
+typedef struct {
+    float *semantic_embedding;                 /* [8192, 256] */
+    tts_hip_host_conv_t input_conv;            /* 292 -> 1024, k 3, s 1 */
+    tts_hip_host_codec_layer_t transformers[8];
+    tts_hip_host_conv_t stage_convs[4];        /* 3 used: transposed 1024 -> 1024, k 4, s 2 */
+    tts_hip_host_conv_t output_proj;           /* 1024 -> 240, k 7, s 1 */
+    float alibi_slopes[8];
+} tts_hip_host_codec_t;
+
 /* ---- exported context (replaces the fields of `g_cuda` that code outside the
  * backend touches: voxtral_tts_cuda.h:51-54,78 read at voxtral_tts_llm.c:380-381) */
 typedef struct {
@@ -204,6 +232,18 @@ void tts_hip_audio_embed(float *out_embed, const int *codes);
  * (host, f32 [36]) -> embedding of the codes written back to d_embed.  Synchronous; returns
  * the codes (END_AUDIO: codes[0] == 1, the rest 2). */
 void tts_hip_generate_frame(int *out_codes, float *d_embed, const float *x0, int pos);
+
+/* Audio codec decoder on the device (the reference runs it on the CPU only).  Upload: codec_ptr
+ * is a tts_codec_t * / tts_hip_host_codec_t * (tts_codec_load fills it, voxtral_tts_codec.c:
+ * 177-270); tensors may be host or device memory; copies.  0 / -1. */
+int tts_hip_upload_codec_weights(void *codec_ptr);
+/* replaces tts_codec_decode (voxtral_tts_codec.c:389-503): host codes [n_frames, 37] ->
+ * *out_samples, a malloc'ed waveform of *out_n_samples = n_frames * 1920 floats that the caller
+ * frees (NULL / 0 on failure); synchronous.  At most 4096 frames per call. */
+void tts_hip_codec_decode(const int *codes, int n_frames, float **out_samples, int *out_n_samples);
+/* The same with device buffers (d_codes [n_frames, 37], d_samples [n_frames * 1920]), queued
+ * on the library's stream without synchronising; 0 / -1. */
+int tts_hip_codec_decode_device(const int *d_codes, int n_frames, float *d_samples);
 
 /* Checkpoint file -> device in one call, in place of the host-side loading that precedes
  * the uploads in the reference (safetensors_open / safetensors_find / safetensors_data,

@@ -71,6 +71,47 @@ typedef struct {
     int n_layers;
 } orc_acoustic_t;
 
+/* Audio codec decoder (voxtral_tts.h:50-58, 66-70, 86-88). */
+#define ORC_CODEC_DIM      1024
+#define ORC_CODEC_HIDDEN   4096
+#define ORC_CODEC_HEADS    8
+#define ORC_CODEC_HEAD_DIM 128
+#define ORC_CODEC_EPS      1e-2f
+#define ORC_CODEC_PATCH    240
+#define ORC_CODEC_SEM_DIM  256
+#define ORC_CODEC_EMBED    292
+#define ORC_CODEC_STAGES   4
+#define ORC_CODEC_LAYERS   8
+
+/* Convolution with its effective weight (voxtral_tts.h:172-180): conv1d [out_ch, in_ch, kernel],
+ * transposed [in_ch, out_ch, kernel]. */
+typedef struct {
+    const float *weight;
+    const float *bias;                   /* [out_ch] or NULL */
+    int in_ch, out_ch, kernel, stride, is_transpose;
+} orc_conv_t;
+
+/* Codec transformer layer (voxtral_tts.h:183-205). */
+typedef struct {
+    const float *wq, *wk, *wv, *wo;      /* f32 [1024,1024] */
+    const float *q_norm, *k_norm;        /* f32 [1024] or NULL */
+    const float *attention_norm;         /* f32 [1024] */
+    const float *w1, *w2, *w3;           /* f32 [4096,1024] [1024,4096] [4096,1024] */
+    const float *ffn_norm;               /* f32 [1024] */
+    const float *attn_scale, *ffn_scale; /* f32 [1024] or NULL */
+    int window_size;
+} orc_codec_layer_t;
+
+/* Codec decoder (voxtral_tts.h:207-225). */
+typedef struct {
+    const float *semantic_embedding;     /* f32 [8192, 256] */
+    orc_conv_t input_conv;               /* 292 -> 1024, k 3 */
+    orc_codec_layer_t layers[ORC_CODEC_LAYERS];
+    orc_conv_t stage_convs[ORC_CODEC_STAGES];   /* 3 used: transposed 1024 -> 1024, k 4, s 2 */
+    orc_conv_t output_proj;              /* 1024 -> 240, k 7 */
+    float alibi_slopes[ORC_CODEC_HEADS];
+} orc_codec_t;
+
 /* Row-parallel worker count for the matvec / linear / attention loops.
  * Rows (and heads) are independent, so results are bit-identical for any
  * count; the reference itself is single-threaded (count 1, the default). */
@@ -132,6 +173,22 @@ void orc_acoustic_forward(const orc_acoustic_t *ac, const float *llm_hidden,
  * (37 rows of a bf16 table, offsets = cumulative unpadded codebook sizes). */
 void orc_audio_embed_forward(const uint16_t *emb_bf16, const int *offsets,
                              const int *codes, float *out_embed, int dim);
+
+/* ---- audio codec decoder (vt_oracle_codec.c) ---- */
+void orc_weight_norm(float *weight, const float *weight_v, const float *weight_g, int out_ch, int fan_in);
+void orc_codec_semantic_embedding(float *emb, const float *emb_sum, const float *cluster_usage);
+void orc_codec_alibi_slopes(float *slopes);
+void orc_linear_f32(float *y, const float *x, const float *W, int seq_len, int in_dim, int out_dim);
+int  orc_causal_conv1d(float *out, const float *in, const float *weight, const float *bias,
+                       int ch_in, int ch_out, int length, int kernel, int stride);
+int  orc_causal_conv_transpose_1d(float *out, const float *in, const float *weight, const float *bias,
+                                  int ch_in, int ch_out, int length, int kernel, int stride);
+void orc_alibi_attention(float *out, const float *Q, const float *K, const float *V, int seq_len,
+                         int n_heads, int n_kv_heads, int head_dim, float scale, int window,
+                         const float *slopes);
+void orc_codec_embed_codes(const float *semantic_embedding, const int *codes, int n_frames, float *out);
+void orc_codec_layer(const orc_codec_layer_t *l, const float *slopes, float *x, int seq);
+int  orc_codec_decode(const orc_codec_t *c, const int *codes, int n_frames, float *out);
 
 #ifdef __cplusplus
 }

@@ -4,7 +4,7 @@ cases.py on the COMPILED REFERENCE (oracle/_ref/libvoxtral_ref.so, built from
 the reference's own sources by `make -C oracle ref`).  The reference tree
 cannot travel, so only the outputs are committed, as .npz data.
 
-    python tests/golden/make_golden.py            # writes kernels/llm/acoustic .npz
+    python tests/golden/make_golden.py            # writes kernels/llm/acoustic/codec .npz
 
 Run it only where the reference tree is mounted.  It also cross-checks the
 oracle bit-for-bit against what it writes and fails loudly on a mismatch.
@@ -18,6 +18,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, HERE)
 import cases  # noqa: E402
+import codec_cases  # noqa: E402
 import vtsupport as S  # noqa: E402
 
 
@@ -32,12 +33,14 @@ def main():
                  "where the reference tree is mounted")
     rb, ob = cases.RefBackend(), cases.OracleBackend(threads=8)
     bad = 0
-    for name, fn in (("kernels", cases.kernel_cases), ("llm", cases.llm_cases),
-                     ("acoustic", cases.acoustic_cases)):
+    crb, cob = codec_cases.RefCodecBackend(), codec_cases.OracleCodecBackend(threads=8)
+    for name, fn, r, o in (("kernels", cases.kernel_cases, rb, ob), ("llm", cases.llm_cases, rb, ob),
+                           ("acoustic", cases.acoustic_cases, rb, ob),
+                           ("codec", codec_cases.codec_cases, crb, cob)):
         t0 = time.time()
-        got = fn(rb)
+        got = fn(r)
         t1 = time.time()
-        mine = fn(ob)
+        mine = fn(o)
         t2 = time.time()
         for k in got:
             if not bit_equal(got[k], mine[k]):

@@ -46,6 +46,26 @@ class HostAcoustic(C.Structure):
                 ("acoustic_out_bf16", vp), ("norm", vp), ("layers", HostLayer * AC_LAYERS)]
 
 
+class HostConv(C.Structure):
+    """tts_hip_host_conv_t == tts_conv_t (voxtral_tts.h:172-180)."""
+    _fields_ = [("weight", vp), ("bias", vp), ("in_ch", C.c_int), ("out_ch", C.c_int),
+                ("kernel", C.c_int), ("stride", C.c_int), ("is_transpose", C.c_int)]
+
+
+class HostCodecLayer(C.Structure):
+    """tts_hip_host_codec_layer_t == tts_codec_layer_t (voxtral_tts.h:183-205)."""
+    _fields_ = [("wq", vp), ("wk", vp), ("wv", vp), ("wo", vp), ("q_norm", vp), ("k_norm", vp),
+                ("attention_norm", vp), ("w1", vp), ("w2", vp), ("w3", vp), ("ffn_norm", vp),
+                ("attn_scale", vp), ("ffn_scale", vp), ("window_size", C.c_int)]
+
+
+class HostCodec(C.Structure):
+    """tts_hip_host_codec_t == tts_codec_t (voxtral_tts.h:207-225)."""
+    _fields_ = [("semantic_embedding", vp), ("input_conv", HostConv),
+                ("transformers", HostCodecLayer * 8), ("stage_convs", HostConv * 4),
+                ("output_proj", HostConv), ("alibi_slopes", C.c_float * 8)]
+
+
 class HipCtx(C.Structure):
     """tts_hip_ctx_t (the exported global g_hip)."""
     _fields_ = [("kv_cache_k_gpu", vp), ("kv_cache_v_gpu", vp), ("kv_cache_max", C.c_int),
@@ -99,6 +119,9 @@ SIGNATURES = {
     "tts_hip_upload_audio_embeddings": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "tts_hip_audio_embed": (None, [C.c_void_p, C.c_void_p]),
     "tts_hip_generate_frame": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]),
+    "tts_hip_upload_codec_weights": (C.c_int, [vp]),
+    "tts_hip_codec_decode": (None, [vp, C.c_int, C.POINTER(f32p), i32p]),
+    "tts_hip_codec_decode_device": (C.c_int, [vp, C.c_int, vp]),
     "tts_hip_load_safetensors": (C.c_int, [C.c_char_p]),
     "tts_hip_safetensors_probe": (C.c_int, [C.c_char_p, C.c_char_p, C.c_char_p, C.c_void_p,
                                             C.c_void_p, C.c_void_p]),

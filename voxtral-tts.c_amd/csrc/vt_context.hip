@@ -153,6 +153,7 @@ static void free_layer(vt_layer_dev *l) {
 extern "C" void tts_hip_free(void) {
     if (!g_vt.initialized) return;
     (void)hipDeviceSynchronize();
+    vt_codec_free();
     for (int i = 0; i < TTS_HIP_DEC_LAYERS; i++) free_layer(&g_vt.h_layers[i]);
     for (int i = 0; i < TTS_HIP_AC_LAYERS; i++) free_layer(&g_vt.ac.layers[i]);
     void *ptrs[] = {g_vt.d_layers, g_vt.d_dec_norm, g_vt.d_tok_emb, g_vt.ac.input_proj,
