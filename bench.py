@@ -318,6 +318,112 @@ def bench_acoustic(args):
     print(json.dumps(out))
 
 
+MFMA_F32_PEAK_TFLOPS = 157.3
+CODEC_FRAMES = 200
+
+
+def codec_flops(frames):
+    """Algorithmic flops of one codec decode: the 8 transformer layers at 1x, 2x, 4x, 8x the frame
+    count (7 products each), the three transposed convolutions, the input and output convolutions
+    (unpadded sizes) and the windowed attention."""
+    d, hid = 1024, 4096
+    total = frames * 2 * (292 * 3) * d
+    for stage, window in enumerate((2, 4, 8, 16)):
+        t = frames << stage
+        total += 2 * t * 2 * (4 * d * d + 3 * d * hid)
+        total += 2 * t * 8 * window * 128 * 4
+        if stage < 3:
+            total += t * 2 * d * d * 4
+    total += (frames * 8) * 2 * d * 240 * 7
+    return total
+
+
+def bench_codec(args):
+    """Codec decoder: 200 frames of 37 codes (16 s of audio) -> 384,000 samples.  A step is one such
+    decode with codes and waveform resident in HBM."""
+    import codecsupport as K
+    import codec_cases as CC
+    Kk, W = args.steps, args.warmup
+    t0 = time.time()
+    hc = K.HostCodec(5)
+    t_gen = time.time() - t0
+    hip = H.Hip(kv_max=8)
+    lib = hip.lib
+    t0 = time.time()
+    cs = hc.struct()
+    assert lib.tts_hip_upload_codec_weights(C.addressof(cs)) == 0, lib.tts_hip_last_error()
+    t_up = time.time() - t0
+    codes = K.random_codes(CODEC_FRAMES, 77)
+    d_codes = H.DevBuf.from_numpy(lib, codes)
+    d_wave = H.DevBuf(lib, CODEC_FRAMES * 1920 * 4)
+    for _ in range(W):
+        assert lib.tts_hip_codec_decode_device(d_codes.ptr, CODEC_FRAMES, d_wave.ptr) == 0
+    lib.tts_hip_sync()
+    lib.tts_hip_timer_start()
+    for _ in range(Kk):
+        lib.tts_hip_codec_decode_device(d_codes.ptr, CODEC_FRAMES, d_wave.ptr)
+    ms_step = lib.tts_hip_timer_stop_ms() / Kk
+    hip.check()
+    wave = d_wave.to_numpy(np.float32, (CODEC_FRAMES * 1920,))
+    shapes = (("qkv 1600x3072x1024", 20, 1600 * 3072 * 1024 * 2), ("wo 1600x1024x1024", 21, 1600 * 1024 * 1024 * 2),
+              ("gate|up 1600x8192x1024", 22, 1600 * 8192 * 1024 * 2), ("down 1600x1024x4096", 23, 1600 * 1024 * 4096 * 2))
+    per_shape = {}
+    for name, which, fl in shapes:
+        ms = lib.tts_hip_bench_kernel(which, 30)
+        per_shape[name] = {"us": round(ms * 1e3, 1), "tflops": round(fl / ms / 1e9, 1)}
+    hip.check()
+    layer_fl = sum(fl for _, _, fl in shapes)
+    layer_ms = sum(v["us"] for v in per_shape.values()) / 1e3
+    achieved = layer_fl / layer_ms / 1e9
+    fl = codec_flops(CODEC_FRAMES)
+    audio_s = CODEC_FRAMES * FRAME_SECONDS
+    out = {
+        "metric": "codec decode ms per 200-frame utterance",
+        "value": round(ms_step, 4), "unit": "ms/utterance",
+        "n_gpus": 1, "steps": Kk, "warmup": W, "ms_per_step": round(ms_step, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "audio codec decoder: 200 frames x 37 codes -> 384,000 samples at 24 kHz (16 s): "
+                               "conv 292->1024, 4 stages of 2 ALiBi sliding-window transformer layers (dim 1024, "
+                               "hidden 4096, windows 2/4/8/16) with 2x transposed convolutions between, conv 1024->240",
+                   "weights": "f32 seeded, weight norm folded", "timed": "events on the library's stream, codes and "
+                   "waveform resident in HBM"},
+        "tflops": round(fl / ms_step / 1e9, 1),
+        "times_real_time": round(audio_s * 1e3 / ms_step, 1),
+        "roofline": {
+            "kernel": "vt_codec_gemm_kernel (the four products of a last-stage layer, 1600 rows)",
+            "bound": "mfma",
+            "achieved": round(achieved, 1), "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(achieved / MFMA_F32_PEAK_TFLOPS, 4),
+            "traffic": measured_traffic("codec"),
+            "flops_per_layer": layer_fl, "ms_per_layer": round(layer_ms, 4), "per_shape": per_shape,
+        },
+        "flops_per_utterance": fl,
+        "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
+        "cpu_baseline": None,
+    }
+    if args.cpu_seconds > 0 and S.have_ref():
+        n = 8
+        b = CC.RefCodecBackend()
+        b.open(hc)
+        t0 = time.time()
+        ref = b.decode(codes[:n])
+        dt = time.time() - t0
+        b.close()
+        got = wave[:n * 1920]
+        # the decoder is causal: the first 8 frames of the long decode equal a decode of 8 frames
+        rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+        out["cpu_baseline"] = {"value": round(dt * 1e3 * CODEC_FRAMES / n, 1), "unit": "ms/utterance", "cores": 1,
+                               "kind": "reference",
+                               "sample": f"tts_codec_decode on the first {n} frames ({dt:.1f} s), scaled by {CODEC_FRAMES // n} "
+                                         "(the cost is linear in the frame count: windowed attention)"}
+        out["parity"] = {"max_abs_over_rms": float(f"{np.abs(ref - got).max() / rms:.3e}"),
+                         "samples_checked": int(ref.size), "against": "reference"}
+        assert np.abs(ref - got).max() / rms < 1e-3
+    hip.close()
+    print(json.dumps(out))
+
+
 AUDIO_ROWS = 8194 + 36 * 23
 FRAME_SECONDS = 0.08                      # one frame of codes is 80 ms of audio (12.5 Hz)
 
@@ -399,7 +505,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=("decode", "prefill", "acoustic", "frame"), default="decode",
+    ap.add_argument("--workload", choices=("decode", "prefill", "acoustic", "frame", "codec"), default="decode",
                     help="decode = the headline metric; prefill / acoustic = the other two configurations")
     ap.add_argument("--mode", type=int, default=0, help="0 persistent kernel, 1 per-phase kernels, 2 streaming kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
@@ -417,6 +523,8 @@ def main():
         return bench_prefill(args)
     if args.workload == "acoustic":
         return bench_acoustic(args)
+    if args.workload == "codec":
+        return bench_codec(args)
     if args.workload == "frame":
         return bench_frame(args)
     K, W = args.steps, args.warmup

@@ -275,7 +275,9 @@ float tts_hip_timer_stop_ms(void);
  * internal stream over `iters` launches on zero-filled work buffers (needs the weights
  * of layer 0 uploaded): which 0..3 = sequence-level product at M = 512 with the q|k|v,
  * output, gate/up and down projection; 4 = causal attention at 512 queries (KV cache of
- * at least 512 rows); 10..13 = the four acoustic phase kernels.  Negative on error. */
+ * at least 512 rows); 10..13 = the four acoustic phase kernels; 20..23 = the codec's fp32
+ * product at 1600 rows with the q|k|v, output, gate|up and down matrices, 24 = the whole codec
+ * decoder on 200 frames (codec weights uploaded).  Negative on error. */
 float tts_hip_bench_kernel(int which, int iters);
 
 #ifdef __cplusplus

@@ -352,6 +352,7 @@ float vt_bench_acoustic_phase(int phase, int iters);
 extern "C" float tts_hip_bench_kernel(int which, int iters) {
     if (!g_vt.initialized || iters < 1) { vt_set_error("tts_hip_bench_kernel: bad call"); return -1.f; }
     if (which >= 10 && which <= 13) return vt_bench_acoustic_phase(which - 10, iters);
+    if (which >= 20 && which <= 24) return vt_bench_codec(which - 20, iters);
     if (which < 0 || which > 4 || g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_bench_kernel: unknown kernel %d", which); return -1.f; }
     const int S = 512;
     if (which == 4 && g_vt.kv_max < S) { vt_set_error("tts_hip_bench_kernel: KV cache shorter than 512"); return -1.f; }

@@ -97,6 +97,7 @@ void vt_launch_add(float *d_a, const float *d_b, int n);
 void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
                                  int q_stride, const float *d_K, const float *d_V, int S, int start_pos);
 void vt_codec_free(void);
+float vt_bench_codec(int which, int iters);
 int vt_stream_supported(void);
 int vt_run_step_stream(const vt_step_args &a);
 int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
