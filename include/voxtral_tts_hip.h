@@ -252,8 +252,9 @@ int tts_hip_codec_decode_device(const int *d_codes, int n_frames, float *d_sampl
  * voxtral_tts_voice.c:251-290).  Maps the .safetensors file and uploads what it holds under
  * the reference's tensor names: backbone layers 0..n-1 (as many consecutive ones as are
  * present) with norm.weight and the token embeddings, the acoustic transformer, the
- * audio-code embedding table.  Returns a bit mask (1 backbone, 2 acoustic, 4 audio-code
- * embeddings) or -1; tts_hip_init first. */
+ * audio-code embedding table, the codec decoder (tts_codec_load, voxtral_tts_codec.c:177-270,
+ * weight norm folded).  Returns a bit mask (1 backbone, 2 acoustic, 4 audio-code embeddings,
+ * 8 codec decoder) or -1; tts_hip_init first. */
 int tts_hip_load_safetensors(const char *path);
 /* Looks one tensor of a .safetensors file up without touching the GPU (safetensors_find,
  * voxtral_tts_safetensors.c:330-345): 0 and dtype (8 chars), rank, shape (4 entries) and

@@ -14,6 +14,9 @@
  *     (oracle/_ref, built from /root/reference by oracle/Makefile) in
  *     tests/test_oracle_vs_ref.py, and frozen in tests/golden/ fixtures
  *     produced by that compiled reference.
+ *   - the codec decoder functions (vt_oracle_codec.c): bit-identical to the compiled
+ *     reference in tests/test_oracle_codec.py, frozen in tests/golden/codec.npz, and
+ *     checked against closed forms and a float64 model of the whole decoder there.
  *   - orc_linear_bf16 with seq_len > 1 follows the reference's no-BLAS
  *     triple loop (voxtral_tts_kernels.c:127-138).  The reference's BLAS
  *     build delegates the summation order to an unpinned third-party

@@ -9,9 +9,9 @@
  * keeps the reference's order, so results do not depend on the worker count.
  *
  * Pin status: every function here is compared bit for bit with the compiled reference sources
- * (oracle/_ref) in tests/golden/make_golden.py and tests/test_oracle_golden.py, frozen in
- * tests/golden/codec_*.npz; closed-form cases (identity convolutions, a window of one, uniform
- * attention) are in tests/test_oracle_math.py.
+ * (oracle/_ref) in tests/golden/make_golden.py and tests/test_oracle_codec.py, frozen in
+ * tests/golden/codec.npz; closed-form cases (delta-tap convolutions, a window of one, geometric
+ * ALiBi weights) and a float64 numpy model of the whole decoder are in tests/test_oracle_codec.py.
  */
 #include "vt_oracle.h"
 

@@ -144,3 +144,68 @@ def test_incomplete_layer_is_an_error(tmp_path):
         assert hip.pkg.ctx().dec_layers_uploaded == 0
     finally:
         hip.close()
+
+
+def test_codec_file_load_equals_struct_upload(tmp_path):
+    """The codec decoder from a file (weight norm folded by the loader, semantic table divided by the
+    cluster usage with its floor: voxtral_tts_codec.c:38-57, 196-205) against the struct upload of
+    arrays prepared by the oracle's restatement of the same steps: waveforms bit-equal."""
+    import ctypes as C
+
+    import codecsupport as K
+    from test_gpu_codec import hip_decode
+
+    o = K.bind_oracle()
+    hc = K.HostCodec(12, distinct_layers=2)
+    usage = (np.abs(S.f32_normal(K.SEM_SIZE, 500, 1.0)) + np.float32(1.0)).astype(np.float32)
+    usage[3] = 0.0                               # floor of 1e-5 applies
+    hc.emb_sum[3] *= np.float32(1e-5)
+    o.orc_codec_semantic_embedding(S.fp(hc.semantic_embedding), S.fp(hc.emb_sum), S.fp(usage))
+
+    t = {"audio_tokenizer.quantizer.semantic_codebook.embedding_sum": torch.from_numpy(hc.emb_sum),
+         "audio_tokenizer.quantizer.semantic_codebook.cluster_usage": torch.from_numpy(usage)}
+
+    def conv(prefix, cv, parametrised=True):
+        if parametrised:
+            shape = (cv.in_ch, cv.out_ch, cv.kernel) if cv.transpose else (cv.out_ch, cv.in_ch, cv.kernel)
+            t[f"{prefix}.conv.parametrizations.weight.original0"] = torch.from_numpy(cv.g).reshape(-1, 1, 1)
+            t[f"{prefix}.conv.parametrizations.weight.original1"] = torch.from_numpy(cv.v).reshape(shape)
+        else:
+            t[f"{prefix}.conv.weight"] = torch.from_numpy(cv.weight)
+        if cv.bias is not None:
+            t[f"{prefix}.conv.bias"] = torch.from_numpy(cv.bias)
+
+    conv("audio_tokenizer.decoder_blocks.0", hc.input_conv)
+    conv("audio_tokenizer.output_proj", hc.output_proj, parametrised=False)
+    for st in range(3):
+        conv(f"audio_tokenizer.decoder_blocks.{2 * st + 2}", hc.stage_convs[st])
+    names = dict(wq="attention.wq.weight", wk="attention.wk.weight", wv="attention.wv.weight",
+                 wo="attention.wo.weight", q_norm="attention.q_norm.weight", k_norm="attention.k_norm.weight",
+                 attention_norm="attention_norm.weight", ffn_norm="ffn_norm.weight", w1="feed_forward.w1.weight",
+                 w2="feed_forward.w2.weight", w3="feed_forward.w3.weight", attn_scale="attention_scale",
+                 ffn_scale="ffn_scale")
+    for i, l in enumerate(hc.layers):
+        for field, suffix in names.items():
+            t[f"audio_tokenizer.decoder_blocks.{2 * (i // 2) + 1}.layers.{i % 2}.{suffix}"] = \
+                torch.from_numpy(getattr(l, field)).clone()     # cycled layers alias: the writer wants copies
+    path = tmp_path / "codec.safetensors"
+    save_file(t, str(path))
+    del t
+
+    codes = K.random_codes(6, 501)
+    codes[4, 0] = 5                              # the row whose usage hit the floor
+    hip = H.Hip(kv_max=8)
+    try:
+        cs = hc.struct()
+        assert hip.lib.tts_hip_upload_codec_weights(C.addressof(cs)) == 0
+        want = hip_decode(hip, codes)
+    finally:
+        hip.close()
+    hip = H.Hip(kv_max=8)
+    try:
+        assert hip.lib.tts_hip_load_safetensors(str(path).encode()) == 8, hip.lib.tts_hip_last_error()
+        got = hip_decode(hip, codes)
+    finally:
+        hip.close()
+    assert np.array_equal(want, got)
+    assert np.isfinite(got).all() and np.abs(got).max() > 0

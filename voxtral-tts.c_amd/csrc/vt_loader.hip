@@ -276,10 +276,100 @@ static int load_layer(const st_file *f, const char *prefix, int i, tts_hip_host_
            l->attention_norm && l->ffn_norm;
 }
 
+/* ---- codec decoder (tts_codec_load, voxtral_tts_codec.c:177-270) ---------------------------- */
+
+struct st_pool { float *p[160]; int n; };
+static float *st_keep(st_pool *pool, float *p) { if (p && pool->n < 160) pool->p[pool->n++] = p; return p; }
+
+/* weight-normed convolution: effective weight = v * g / |v| per row (voxtral_tts_codec.c:38-57,
+ * 71-119), or the plain .conv.weight of a checkpoint without the parametrisation */
+static int load_conv(const st_file *f, st_pool *pool, const char *prefix, tts_hip_host_conv_t *cv, int in_ch,
+                     int out_ch, int kernel, int stride, int transpose) {
+    char name[256];
+    const int rows = transpose ? in_ch : out_ch, fan_in = (transpose ? out_ch : in_ch) * kernel;
+    const long long n = (long long)rows * fan_in;
+    snprintf(name, sizeof name, "%s.conv.parametrizations.weight.original0", prefix);
+    float *g = st_f32(f, name, rows);
+    snprintf(name, sizeof name, "%s.conv.parametrizations.weight.original1", prefix);
+    float *v = st_f32(f, name, n);
+    if (g && v) {
+        for (int o = 0; o < rows; o++) {
+            float *row = v + (size_t)o * fan_in;
+            float nsq = 0.0f;
+            for (int i = 0; i < fan_in; i++) nsq += row[i] * row[i];
+            const float scale = g[o] / sqrtf(nsq + 1e-12f);
+            for (int i = 0; i < fan_in; i++) row[i] *= scale;
+        }
+        free(g);
+        cv->weight = st_keep(pool, v);
+    } else {
+        free(g); free(v);
+        snprintf(name, sizeof name, "%s.conv.weight", prefix);
+        cv->weight = st_keep(pool, st_f32(f, name, n));
+    }
+    snprintf(name, sizeof name, "%s.conv.bias", prefix);
+    cv->bias = st_keep(pool, st_f32(f, name, out_ch));
+    cv->in_ch = in_ch; cv->out_ch = out_ch; cv->kernel = kernel; cv->stride = stride; cv->is_transpose = transpose;
+    return cv->weight != NULL;
+}
+
+static int load_codec(const st_file *f, const char *path) {
+    tts_hip_host_codec_t *c = (tts_hip_host_codec_t *)calloc(1, sizeof *c);
+    st_pool pool;
+    pool.n = 0;
+    int ok = c != NULL, rc = -1;
+    char name[256];
+    if (ok) {
+        float *sum = st_f32(f, "audio_tokenizer.quantizer.semantic_codebook.embedding_sum", 8192LL * 256);
+        float *usage = st_f32(f, "audio_tokenizer.quantizer.semantic_codebook.cluster_usage", 8192);
+        ok = sum && usage;
+        for (int i = 0; ok && i < 8192; i++) {
+            const float u = usage[i] < 1e-5f ? 1e-5f : usage[i];
+            for (int j = 0; j < 256; j++) sum[i * 256 + j] /= u;
+        }
+        free(usage);
+        c->semantic_embedding = st_keep(&pool, sum);
+        for (int h = 0; h < 8; h++) c->alibi_slopes[h] = powf(2.0f, -8.0f / 8.0f * (float)(h + 1));
+    }
+    ok = ok && load_conv(f, &pool, "audio_tokenizer.decoder_blocks.0", &c->input_conv, 292, 1024, 3, 1, 0);
+    static const int windows[4] = {2, 4, 8, 16};
+    int block = 1;
+    for (int stage = 0; ok && stage < 4; stage++) {
+        for (int l = 0; ok && l < 2; l++) {
+            tts_hip_host_codec_layer_t *L = &c->transformers[stage * 2 + l];
+#define VT_CT(field, suffix, count) \
+            (snprintf(name, sizeof name, "audio_tokenizer.decoder_blocks.%d.layers.%d." suffix, block, l), \
+             L->field = st_keep(&pool, st_f32(f, name, count)))
+            VT_CT(wq, "attention.wq.weight", 1024LL * 1024); VT_CT(wk, "attention.wk.weight", 1024LL * 1024);
+            VT_CT(wv, "attention.wv.weight", 1024LL * 1024); VT_CT(wo, "attention.wo.weight", 1024LL * 1024);
+            VT_CT(q_norm, "attention.q_norm.weight", 1024); VT_CT(k_norm, "attention.k_norm.weight", 1024);
+            VT_CT(attention_norm, "attention_norm.weight", 1024); VT_CT(ffn_norm, "ffn_norm.weight", 1024);
+            VT_CT(w1, "feed_forward.w1.weight", 4096LL * 1024); VT_CT(w2, "feed_forward.w2.weight", 1024LL * 4096);
+            VT_CT(w3, "feed_forward.w3.weight", 4096LL * 1024);
+            VT_CT(attn_scale, "attention_scale", 1024); VT_CT(ffn_scale, "ffn_scale", 1024);
+#undef VT_CT
+            L->window_size = windows[stage];
+            ok = L->wq && L->wk && L->wv && L->wo && L->attention_norm && L->ffn_norm && L->w1 && L->w2 && L->w3;
+        }
+        block++;
+        if (ok && stage < 3) {
+            snprintf(name, sizeof name, "audio_tokenizer.decoder_blocks.%d", block);
+            ok = load_conv(f, &pool, name, &c->stage_convs[stage], 1024, 1024, 4, 2, 1);
+            block++;
+        }
+    }
+    ok = ok && load_conv(f, &pool, "audio_tokenizer.output_proj", &c->output_proj, 1024, 240, 7, 1, 0);
+    if (!ok) vt_set_error("safetensors: codec decoder of %s is incomplete", path);
+    else rc = tts_hip_upload_codec_weights(c);
+    for (int i = 0; i < pool.n; i++) free(pool.p[i]);
+    free(c);
+    return rc;
+}
+
 /* Uploads what the file holds under the reference's tensor names: backbone layers 0..n-1 (as
  * many consecutive ones as are present, at most 26) with norm.weight, the acoustic
- * transformer (all of it or none), the audio-code embedding table.  Returns a bit mask
- * (1 backbone, 2 acoustic, 4 audio embeddings; the number of backbone layers is in
+ * transformer (all of it or none), the audio-code embedding table, the codec decoder.  Returns a
+ * bit mask (1 backbone, 2 acoustic, 4 audio embeddings, 8 codec decoder; the number of backbone layers is in
  * g_hip.dec_layers_uploaded) or -1.  tts_hip_init must have been called. */
 extern "C" int tts_hip_load_safetensors(const char *path) {
     if (!g_vt.initialized) { vt_set_error("tts_hip_load_safetensors: backend not initialised"); return -1; }
@@ -358,6 +448,10 @@ extern "C" int tts_hip_load_safetensors(const char *path) {
             else if (tts_hip_upload_audio_embeddings(emb, (int)rows, offs) == 0) mask |= 4;
             else rc = -1;
         }
+    }
+    if (!rc && st_find(&f, "audio_tokenizer.quantizer.semantic_codebook.embedding_sum")) {
+        if (load_codec(&f, path) == 0) mask |= 8;
+        else rc = -1;
     }
     for (int i = 0; i < nfree; i++) free(tofree[i]);
     st_close(&f);
