@@ -21,9 +21,12 @@ def assert_close(ref, got, what, tol=TOL):
     return mx, l2
 
 
-def test_one_layer_decode_with_512_cached_positions():
-    """Config 2: one layer, batch 1, KV cache of 512 positions ~N(0,1), hidden ~N(0,1), pos = 512."""
-    kv_max, pos = 520, 512
+@pytest.mark.parametrize("pos", [512, 511, 300, 129, 128, 33, 1])
+def test_one_layer_decode_with_cached_positions(pos):
+    """Config 2: one layer, batch 1, KV cache of 512 positions ~N(0,1), hidden ~N(0,1), pos = 512;
+    shorter caches take the attention schedule with one workgroup per query head (up to 511
+    cached positions, in batches of 128), 512 and more the chunked one."""
+    kv_max = 520
     layer = S.Layer(3)
     ones = np.ones(S.DIM, np.float32)
     k = np.zeros((26, kv_max, S.KV_DIM), np.float32)

@@ -290,7 +290,103 @@ __device__ __forceinline__ void vt_attn_geometry(int n, int nch_max, int nw, int
     nch = (n + cs - 1) / cs;
 }
 
+/* Short caches (at most VT_ATT_DIRECT_MAX positions): one workgroup per QUERY head, no
+ * cross-workgroup merge and so no store / counter / reload round trips inside the phase.
+ * Lanes 16g..16g+15 of a wave serve position slot g and own 8 of the 128 dims, so a wave
+ * works on 4 positions at once and the workgroup on 32; a batch of 4 such rounds (128
+ * positions) has all its K and V rows requested before any is used.  Each of the 32 lane
+ * groups keeps its own online-softmax state; they are merged through LDS at the end.  The
+ * four workgroups of a kv head sit on one XCD (blockIdx % 8) and share its rows in that L2. */
+#define VT_ATT_DIRECT_MAX 512
+
+/* K and V rows of one batch: 4 rounds of one position per lane group */
+struct vt_att_rows { f32x4 ka[4], kb[4], va[4], vb[4]; };
+
+__device__ __forceinline__ bool vt_attn_is_direct(const vt_step_args &a) {
+    return a.pos < VT_ATT_DIRECT_MAX && (int)gridDim.x >= VT_HEADS;
+}
+
+/* Requests the rows jb, jb + stride, ... of kv head kvh (clamped to `last`; rows beyond it are
+ * loaded but never used). */
+__device__ __forceinline__ void vt_attn_fetch(vt_att_rows &r, const vt_step_args &a, int layer, int kvh,
+                                              int jb, int stride, int last) {
+    const int sub = vt_lane() & 15;
+    const size_t off = (size_t)(a.first_layer + layer) * a.kv_max * VT_KV_DIM + kvh * VT_HEAD_DIM + sub * 8;
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int j = max(min(jb + u * stride, last), 0);
+        const f32x4 *kp = reinterpret_cast<const f32x4 *>(a.kv_k + off + (size_t)j * VT_KV_DIM);
+        const f32x4 *vp = reinterpret_cast<const f32x4 *>(a.kv_v + off + (size_t)j * VT_KV_DIM);
+        r.ka[u] = kp[0]; r.kb[u] = kp[1];
+        r.va[u] = vp[0]; r.vb[u] = vp[1];
+    }
+}
+
+struct vt_att_state { float m, l; f32x4 oa, ob; };
+
+__device__ __forceinline__ void vt_attn_step(vt_att_state &st, const f32x4 &qa, const f32x4 &qb, const f32x4 &ka,
+                                             const f32x4 &kb, const f32x4 &va, const f32x4 &vb, float scale) {
+    float s = qa.x * ka.x;
+    s = fmaf(qa.y, ka.y, s); s = fmaf(qa.z, ka.z, s); s = fmaf(qa.w, ka.w, s);
+    s = fmaf(qb.x, kb.x, s); s = fmaf(qb.y, kb.y, s); s = fmaf(qb.z, kb.z, s);
+    s = fmaf(qb.w, kb.w, s);
+    s = vt_row16_sum(s) * scale;
+    const float mn = fmaxf(st.m, s);
+    const float corr = __expf(st.m - mn), p = __expf(s - mn);
+    st.l = fmaf(st.l, corr, p);
+    st.oa = st.oa * corr + va * p;
+    st.ob = st.ob * corr + vb * p;
+    st.m = mn;
+}
+
+__device__ __forceinline__ void vt_attn_direct(const vt_step_args &a, int layer, float *lds) {
+    const int wg = (int)blockIdx.x;
+    if (wg >= VT_HEADS) return;
+    const int kvh = wg % VT_KV_HEADS, head = kvh * 4 + wg / VT_KV_HEADS;
+    const int nw = (int)(blockDim.x >> 6), wave = vt_wave(), lane = vt_lane();
+    const int grp = lane >> 4, sub = lane & 15;
+    const int slot = wave * 4 + grp, nslot = nw * 4;
+    const int n = a.pos + 1;
+    const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
+    const f32x4 qa = vt_ldc4(a.q, (head * VT_HEAD_DIM + sub * 8) / 4, VT_Q_DIM);
+    const f32x4 qb = vt_ldc4(a.q, (head * VT_HEAD_DIM + sub * 8) / 4 + 1, VT_Q_DIM);
+    vt_att_state st = {-1e30f, 0.f, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    for (int jb = slot; jb < n; jb += 4 * nslot) {
+        vt_att_rows r;
+        vt_attn_fetch(r, a, layer, kvh, jb, nslot, n - 1);
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+            if (jb + u * nslot < n) vt_attn_step(st, qa, qb, r.ka[u], r.kb[u], r.va[u], r.vb[u], scale);
+    }
+
+    /* merge the lane groups of the workgroup: idle slots hold (m = -1e30, l = 0, o = 0) */
+    float *mine = lds + slot * VT_ATT_STRIDE;                  /* [nslot][VT_ATT_STRIDE] */
+    if (sub == 0) { mine[0] = st.m; mine[1] = st.l; }
+    *reinterpret_cast<f32x4 *>(mine + 4 + sub * 8) = st.oa;
+    *reinterpret_cast<f32x4 *>(mine + 8 + sub * 8) = st.ob;
+    __syncthreads();
+    float *wgt = lds + nslot * VT_ATT_STRIDE;                  /* [nslot] weights exp(m_s - M) */
+    if (wave == 0) {
+        const float ms = lane < nslot ? lds[lane * VT_ATT_STRIDE] : -1e30f;
+        float M = vt_row16_max(ms);
+        M = fmaxf(fmaxf(vt_readlane(M, 0), vt_readlane(M, 16)), fmaxf(vt_readlane(M, 32), vt_readlane(M, 48)));
+        if (lane < nslot) wgt[lane] = __expf(ms - M);
+    }
+    __syncthreads();
+    const int d = (int)threadIdx.x;
+    if (d < VT_HEAD_DIM) {
+        float Ls = 0.f, O = 0.f;
+        for (int w = 0; w < nslot; w++) {
+            const float e = wgt[w];
+            Ls = fmaf(lds[w * VT_ATT_STRIDE + 1], e, Ls);
+            O = fmaf(lds[w * VT_ATT_STRIDE + 4 + d], e, O);
+        }
+        vt_stc(a.attn + head * VT_HEAD_DIM + d, O * (1.0f / Ls));
+    }
+}
+
 __device__ __forceinline__ void vt_attn_phase(const vt_step_args &a, int layer, float *lds) {
+    if (vt_attn_is_direct(a)) { vt_attn_direct(a, layer, lds); return; }
     const int G = (int)gridDim.x;
     const int nch_max = G / VT_KV_HEADS;
     const int wg = (int)blockIdx.x;
