@@ -72,9 +72,14 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
         vt_qkv_body(ring, L, a, l, x_in, lds, [&] { vt_wo_prefetch(ring, L, VT_PART_HEAD); });
         if (!vt_barrier_then(gs, &s_flag, [&] { vt_wo_prefetch(ring, L, VT_PART_TAIL); }, tn)) return;
         vt_attn_phase(a, l, lds);
-        if (!vt_barrier_then(gs, &s_flag, [] {}, tn)) return;
-        vt_wo_body(ring, L, a, x_in, lds, [&] { vt_w13_prefetch(ring, L, VT_PART_HEAD); });
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L, VT_PART_TAIL); }, tn)) return;
+        /* with 3 rows per wave the output projection leaves the ring slots from VT_WO_SLOTS on
+         * free: the gate|up rows that go there are requested a phase early */
+        const int wo_slots = vt_wo_rows().nr * 4 <= VT_WO_SLOTS ? VT_WO_SLOTS : VT_RING;
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L, VT_PART_ALL, wo_slots, VT_RING); }, tn))
+            return;
+        vt_wo_body(ring, L, a, x_in, lds, [&] { vt_w13_prefetch(ring, L, VT_PART_HEAD, 0, wo_slots); });
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L, VT_PART_TAIL, 0, wo_slots); }, tn))
+            return;
         vt_w13_body(ring, L, a, lds, [&] { vt_w2_prefetch(ring, L, VT_PART_HEAD); });
         if (!vt_barrier_then(gs, &s_flag, [&] { vt_w2_prefetch(ring, L, VT_PART_TAIL); }, tn)) return;
         vt_w2_body(ring, L, a, lds, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1], VT_PART_HEAD); });

@@ -174,9 +174,12 @@ __device__ __forceinline__ vt_rows vt_split_rows(int n_rows, int align, int k_pe
 enum { VT_PART_ALL = 0, VT_PART_HEAD = 1, VT_PART_TAIL = 2 };
 #define VT_HEAD_SLOTS 6        /* ring slots (KB per wave) requested ahead of the hand-over */
 
+/* Only the ring slots [slot_lo, slot_hi) are requested: the output projection leaves the last 6
+ * slots of the ring unused, so the gate|up rows that live there are requested a phase early. */
 template <int NK, int D>
 __device__ __forceinline__ void vt_ring_prefetch(u32x4 (&ring)[VT_RING], const uint16_t *W,
-                                                 int row_len, const vt_rows &r, int part = VT_PART_ALL) {
+                                                 int row_len, const vt_rows &r, int part = VT_PART_ALL,
+                                                 int slot_lo = 0, int slot_hi = VT_RING) {
     static_assert(NK * D <= VT_RING, "ring too small");
     const uint16_t *base = W + (size_t)r.r0 * row_len + r.kofs + vt_lane() * 8;
 #pragma unroll
@@ -184,9 +187,10 @@ __device__ __forceinline__ void vt_ring_prefetch(u32x4 (&ring)[VT_RING], const u
         if (j < r.nr) {
 #pragma unroll
             for (int c = 0; c < NK; c++) {
-                const bool head = j * NK + c < VT_HEAD_SLOTS;
-                if (part == VT_PART_ALL || (part == VT_PART_HEAD) == head)
-                    ring[j * NK + c] = vt_ldw(base + (size_t)j * row_len + c * 512);
+                const int slot = j * NK + c;
+                const bool head = slot - slot_lo < VT_HEAD_SLOTS;
+                if (slot >= slot_lo && slot < slot_hi && (part == VT_PART_ALL || (part == VT_PART_HEAD) == head))
+                    ring[slot] = vt_ldw(base + (size_t)j * row_len + c * 512);
             }
         }
     }
@@ -540,9 +544,11 @@ __device__ __forceinline__ void vt_wo_body(u32x4 (&ring)[VT_RING], const vt_laye
 
 __device__ __forceinline__ vt_rows vt_w13_rows() { return vt_split_rows<1>(2 * VT_FFN, 2, 0); }
 
+#define VT_WO_SLOTS 12         /* ring slots the output projection uses (3 rows x 4 KB per wave) */
+
 __device__ __forceinline__ void vt_w13_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
-                                                int part = VT_PART_ALL) {
-    vt_ring_prefetch<6, 3>(ring, L.w13, VT_DIM, vt_w13_rows(), part);
+                                                int part = VT_PART_ALL, int slot_lo = 0, int slot_hi = VT_RING) {
+    vt_ring_prefetch<6, 3>(ring, L.w13, VT_DIM, vt_w13_rows(), part, slot_lo, slot_hi);
 }
 
 template <class AR = vt_nothing>
