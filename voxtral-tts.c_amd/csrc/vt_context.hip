@@ -126,7 +126,7 @@ extern "C" int tts_hip_init(int kv_cache_max) {
         {(void **)&g_vt.d_att_cnt, sizeof(unsigned) * TTS_HIP_DEC_LAYERS * VT_KV_HEADS},
         {(void **)&g_vt.d_embed, sizeof(float) * VT_DIM},
         {(void **)&g_vt.d_hidden, sizeof(float) * (VT_DIM + 64)},
-        {(void **)&g_vt.d_bar_flags, sizeof(unsigned) * (size_t)g_vt.grid + 256},
+        {(void **)&g_vt.d_bar_flags, sizeof(unsigned) * (size_t)VT_FLAG_COPIES * VT_FLAG_STRIDE},
         {(void **)&g_vt.d_abort, 256},
         {(void **)&g_vt.d_dummy, 4096},
     };

@@ -152,11 +152,12 @@ vt_final_kernel(vt_step_args a) {
 
 /* ---- host side ------------------------------------------------------------------- */
 
-/* Rows per workgroup of every phase must fit the 256-float LDS row buffer. */
+/* Rows per workgroup of every phase must fit the 256-float LDS row buffer, and a lane of the
+ * barrier polls VT_FLAG_LOADS flags. */
 static int grid_fits(int grid) {
     int per = (2 * VT_FFN + grid - 1) / grid;
     per = (per + 1) / 2 * 2;
-    return per <= 256 && grid % VT_KV_HEADS == 0 && grid >= VT_KV_HEADS;
+    return per <= 256 && grid % VT_KV_HEADS == 0 && grid >= VT_KV_HEADS && grid <= VT_WAVE * VT_FLAG_LOADS;
 }
 
 int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
@@ -234,7 +235,7 @@ static int step_aborted(int flag) {
     if (!flag) return 0;
     vt_set_error("decode step: grid barrier timed out; kernel left early, result invalid");
     (void)hipMemsetAsync(g_vt.d_abort, 0, sizeof(int), g_vt.stream);
-    (void)hipMemsetAsync(g_vt.d_bar_flags, 0, sizeof(unsigned) * g_vt.grid, g_vt.stream);
+    (void)hipMemsetAsync(g_vt.d_bar_flags, 0, sizeof(unsigned) * VT_FLAG_COPIES * VT_FLAG_STRIDE, g_vt.stream);
     (void)hipStreamSynchronize(g_vt.stream);
     g_vt.bar_epoch = 0;
     return -1;

@@ -154,24 +154,57 @@ struct vt_grid_sync {
     unsigned long long timeout;     /* wall_clock64 ticks (100 MHz) */
 };
 
+/* The flags exist in VT_FLAG_COPIES copies, VT_FLAG_STRIDE words apart (so in different memory
+ * channels); a workgroup writes all copies and polls copy blockIdx % VT_FLAG_COPIES: the polls
+ * of 256 workgroups are coherent loads served by the memory side, and spread over the copies
+ * they do not queue on one channel. */
+#define VT_FLAG_COPIES 8
+#define VT_FLAG_STRIDE 16384
+#define VT_FLAG_LOADS 4           /* flags a lane polls: grids of up to 256 workgroups */
+#ifndef VT_POLL_DEPTH
+#define VT_POLL_DEPTH 2
+#endif
+
 __device__ __forceinline__ void vt_barrier_arrive(vt_grid_sync &gs) {
     __builtin_amdgcn_s_waitcnt(0x0F70);          /* vmcnt(0): this wave's stores are acknowledged */
     __syncthreads();
-    if (threadIdx.x == 0) vt_stc_u32(gs.flags + blockIdx.x, gs.epoch);
+    if (threadIdx.x < VT_FLAG_COPIES) vt_stc_u32(gs.flags + threadIdx.x * VT_FLAG_STRIDE + blockIdx.x, gs.epoch);
 }
 
 __device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag) {
     if (threadIdx.x < VT_WAVE) {
         const int G = (int)gridDim.x;
+        const unsigned *mine = gs.flags + (blockIdx.x % VT_FLAG_COPIES) * VT_FLAG_STRIDE;
         const unsigned long long t0 = wall_clock64();
         int ok = 1;
-        for (;;) {
-            int done = 1;
-            for (int i = (int)threadIdx.x; i < G; i += VT_WAVE)
-                done &= (int)(vt_ldc_u32(gs.flags + i) - gs.epoch) >= 0;
-            if (__all(done)) break;
-            if (__hip_atomic_load(gs.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
-                wall_clock64() - t0 > gs.timeout) {
+        /* VT_POLL_DEPTH polls are kept in flight, so the release is seen a fraction of a memory
+         * latency after it could be.  A lane reads the flags lane, lane + 64, ... (the last one
+         * again where the grid has fewer). */
+        const int lane = (int)threadIdx.x;
+        unsigned f[VT_POLL_DEPTH][VT_FLAG_LOADS];
+#pragma unroll
+        for (int d = 0; d < VT_POLL_DEPTH; d++)
+#pragma unroll
+            for (int k = 0; k < VT_FLAG_LOADS; k++) f[d][k] = vt_ldc_u32(mine + min(lane + VT_WAVE * k, G - 1));
+        bool released = false;
+        while (!released) {
+            /* the abort flag travels with the flags: one round trip per poll, not two */
+            const int aborted = __hip_atomic_load(gs.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int d = 0; d < VT_POLL_DEPTH; d++) {
+                if (!released) {
+                    int done = 1;
+#pragma unroll
+                    for (int k = 0; k < VT_FLAG_LOADS; k++) done &= (int)(f[d][k] - gs.epoch) >= 0;
+                    released = __all(done);
+                    if (!released) {
+#pragma unroll
+                        for (int k = 0; k < VT_FLAG_LOADS; k++)
+                            f[d][k] = vt_ldc_u32(mine + min(lane + VT_WAVE * k, G - 1));
+                    }
+                }
+            }
+            if (!released && (aborted != 0 || wall_clock64() - t0 > gs.timeout)) {
                 ok = 0;
                 break;
             }
