@@ -27,8 +27,12 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 #define VT_FFN      9216
 #define VT_EPS      1e-5f
 
-__device__ __forceinline__ int vt_lane() { return (int)(threadIdx.x & (VT_WAVE - 1)); }
-__device__ __forceinline__ int vt_wave() { return (int)(threadIdx.x >> 6); }
+/* The thread index goes through an empty asm: what a phase of a persistent kernel derives from
+ * it (lane offsets, row pointers) is then recomputed where it is used instead of being hoisted
+ * out of the layer loop and kept in registers, or in scratch, for the whole kernel. */
+__device__ __forceinline__ int vt_tid() { int t = (int)threadIdx.x; asm volatile("" : "+v"(t)); return t; }
+__device__ __forceinline__ int vt_lane() { return vt_tid() & (VT_WAVE - 1); }
+__device__ __forceinline__ int vt_wave() { return vt_tid() >> 6; }
 
 /* bf16 pair packed in a dword: element 0 in the low half. Widening is exact. */
 __device__ __forceinline__ float vt_bf16_lo(unsigned int w) { return __uint_as_float(w << 16); }
