@@ -172,7 +172,9 @@ __device__ __forceinline__ vt_rows vt_split_rows(int n_rows, int align, int k_pe
  * 48 KB per CU, about what a CU accepts as outstanding loads; more would hold up the
  * acknowledgement of the hand-over stores that the barrier waits for. */
 enum { VT_PART_ALL = 0, VT_PART_HEAD = 1, VT_PART_TAIL = 2 };
+#ifndef VT_HEAD_SLOTS
 #define VT_HEAD_SLOTS 6        /* ring slots (KB per wave) requested ahead of the hand-over */
+#endif
 
 /* Only the ring slots [slot_lo, slot_hi) are requested: the output projection leaves the last 6
  * slots of the ring unused, so the gate|up rows that live there are requested a phase early. */
