@@ -265,6 +265,10 @@ int tts_hip_safetensors_probe(const char *path, const char *name, char *dtype8, 
 /* Decode schedule: 0 = persistent whole-step kernel (default), 1 = one kernel per
  * phase, 2 = streaming whole-step kernel (256-CU devices; experimental). */
 void tts_hip_set_decode_mode(int mode);
+/* Spin budget of one grid barrier of the whole-step kernels, in ticks of the 100 MHz wall clock
+ * (0 = the default of 0.2 s).  When it runs out every workgroup leaves the kernel, the call
+ * reports an error and the result is invalid; the next call starts clean. */
+void tts_hip_set_barrier_timeout(unsigned long long ticks);
 /* Number of failed calls since init, and the text of the last failure. */
 int tts_hip_error_count(void);
 const char *tts_hip_last_error(void);

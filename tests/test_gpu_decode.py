@@ -156,3 +156,33 @@ def test_position_outside_cache_is_an_error_not_a_fault():
         assert b"outside the KV cache" in hip.lib.tts_hip_last_error()
     finally:
         hip.close()
+
+
+def test_barrier_budget_exhausted_is_reported_and_recoverable():
+    """The grid barrier spins against a wall-clock budget.  With a budget of one tick the
+    first unfinished poll gives up: every workgroup leaves the kernel, the call is counted as
+    failed, and with the default budget back the same step runs and matches the oracle."""
+    layers = [S.Layer(1)]
+    ones = np.ones(S.DIM, np.float32)
+    orc = cases.OracleBackend(threads=16)
+    orc.llm_open(layers, ones, 16, n_layers=4)
+    e = S.f32_normal(S.DIM, 6)
+    ref = orc.llm_forward(e)
+    hip = H.Hip(kv_max=16)
+    try:
+        hip.upload_decoder(layers, ones, 4)
+        lib = hip.lib
+        n0 = lib.tts_hip_error_count()
+        lib.tts_hip_set_barrier_timeout(1)
+        out = np.zeros(S.DIM, np.float32)
+        lib.tts_hip_llm_forward(out.ctypes.data, e.ctypes.data, 0)
+        assert lib.tts_hip_error_count() == n0 + 1
+        assert b"barrier timed out" in lib.tts_hip_last_error()
+        lib.tts_hip_set_barrier_timeout(0)
+        hip.err0 = lib.tts_hip_error_count()
+        hip.pos = 0
+        got = hip.llm_forward(e)
+        assert_close(ref, got, "after the timed-out step")
+    finally:
+        hip.lib.tts_hip_set_barrier_timeout(0)
+        hip.close()

@@ -331,6 +331,7 @@ extern "C" void tts_hip_sync(void) {
 }
 
 extern "C" void tts_hip_set_decode_mode(int mode) { g_vt.decode_mode = mode; }
+extern "C" void tts_hip_set_barrier_timeout(unsigned long long ticks) { g_vt.bar_timeout = ticks; }
 extern "C" int tts_hip_error_count(void) { return g_vt.error_count; }
 extern "C" const char *tts_hip_last_error(void) { return g_vt.last_error; }
 

@@ -202,7 +202,7 @@ int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
         gs.flags = g_vt.d_bar_flags;
         gs.abort_flag = g_vt.d_abort;
         gs.epoch = g_vt.bar_epoch + 1u;
-        gs.timeout = 20000000ull;                 /* 0.2 s of the 100 MHz wall clock */
+        gs.timeout = g_vt.bar_timeout ? g_vt.bar_timeout : 20000000ull;   /* default 0.2 s of the 100 MHz wall clock */
         g_vt.bar_epoch += 5u * (unsigned)n_layers;
         static int attr_set = 0;
         if (!attr_set && g_vt.step_dyn_lds) {

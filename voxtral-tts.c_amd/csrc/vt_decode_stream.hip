@@ -634,7 +634,7 @@ int vt_run_step_stream(const vt_step_args &a) {
     gs.flags = g_vt.d_bar_flags;
     gs.abort_flag = g_vt.d_abort;
     gs.epoch = g_vt.bar_epoch + 1u;
-    gs.timeout = 20000000ull;                       /* 0.2 s of the 100 MHz wall clock */
+    gs.timeout = g_vt.bar_timeout ? g_vt.bar_timeout : 20000000ull;   /* default 0.2 s of the 100 MHz wall clock */
     g_vt.bar_epoch += 5u * (unsigned)a.n_layers;
     hipLaunchKernelGGL(vt_decode_stream_kernel, dim3(g_vt.grid), dim3(VS_THREADS), dyn, g_vt.stream,
                        a, gs, (const uint16_t *)g_vt.d_dummy);

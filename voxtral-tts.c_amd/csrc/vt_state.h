@@ -64,6 +64,7 @@ struct vt_state {
     unsigned int *d_att_cnt;
     unsigned int *d_bar_flags;    /* one flag per workgroup of the persistent kernel */
     unsigned int bar_epoch;       /* last barrier epoch handed to a launch */
+    unsigned long long bar_timeout; /* spin budget of a barrier in 100 MHz ticks; 0 = default */
     int *d_abort;
     uint16_t *d_dummy;            /* small resident block requested in place of a layer beyond the last */
     float *h_pin;                 /* pinned staging: [3072 in][3072 out + flag] */
