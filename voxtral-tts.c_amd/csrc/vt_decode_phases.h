@@ -391,6 +391,30 @@ __device__ __forceinline__ void vt_attn_direct(const vt_step_args &a, int layer,
     }
 }
 
+/* While a layer's attention runs on 32 workgroups, the others pull the K and V rows that the
+ * NEXT layer's attention will read into the L2 of the XCD that will read them (kv head =
+ * blockIdx % 8, one lane per 128-byte line, plain loads).  The rows are small (1 KB per position
+ * and kv head) and nothing else allocates in L2 in between - weights stream with the
+ * non-temporal hint - so the next attention finds them there instead of in HBM.  Wave 0 stays
+ * out of it: it polls the barrier. */
+__device__ __forceinline__ void vt_kv_l2_prefetch(const vt_step_args &a, int layer) {
+    const int G = (int)gridDim.x, wg = (int)blockIdx.x, nw = (int)(blockDim.x >> 6);
+    if ((G & 7) || wg < VT_HEADS || vt_wave() == 0) return;
+    const int idle0 = VT_HEADS >> 3;                            /* workgroups per XCD that run the attention */
+    const int me = (((wg >> 3) - idle0) * (nw - 1) + vt_wave() - 1) * VT_WAVE + vt_lane();
+    const int n_lanes = ((G >> 3) - idle0) * (nw - 1) * VT_WAVE;
+    const int lines_per_row = VT_HEAD_DIM * 4 / 128;            /* 4 */
+    const int total = 2 * a.pos * lines_per_row;                /* K and V rows 0 .. pos - 1 */
+    const size_t base = (size_t)(a.first_layer + layer) * a.kv_max * VT_KV_DIM + (wg & 7) * VT_HEAD_DIM;
+    unsigned acc = 0u;
+    for (int g = me; g < total; g += n_lanes) {
+        const int line = g % lines_per_row, row = (g / lines_per_row) % a.pos, kv = g / (lines_per_row * a.pos);
+        const float *p = (kv ? a.kv_v : a.kv_k) + base + (size_t)row * VT_KV_DIM + line * 32;
+        acc ^= *reinterpret_cast<const unsigned *>(p);
+    }
+    asm volatile("" ::"v"(acc));
+}
+
 __device__ __forceinline__ void vt_attn_phase(const vt_step_args &a, int layer, float *lds) {
     if (vt_attn_is_direct(a)) { vt_attn_direct(a, layer, lds); return; }
     const int G = (int)gridDim.x;
