@@ -77,7 +77,10 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
         const int wo_slots = vt_wo_rows().nr * 4 <= VT_WO_SLOTS ? VT_WO_SLOTS : VT_RING;
         if (!vt_barrier_then(gs, &s_flag, [&] {
                 vt_w13_prefetch(ring, L, VT_PART_ALL, wo_slots, VT_RING);
-                if (more && vt_attn_is_direct(a)) vt_kv_l2_prefetch(a, l + 1);
+                if (vt_attn_is_direct(a)) {
+                    vt_w13_l2_prefetch(L);
+                    if (more) vt_kv_l2_prefetch(a, l + 1);
+                }
             }, tn))
             return;
         vt_wo_body(ring, L, a, x_in, lds, [&] { vt_w13_prefetch(ring, L, VT_PART_HEAD, 0, wo_slots); });

@@ -577,6 +577,34 @@ __device__ __forceinline__ void vt_w13_prefetch(u32x4 (&ring)[VT_RING], const vt
     vt_ring_prefetch<6, 3>(ring, L.w13, VT_DIM, vt_w13_rows(), part, slot_lo, slot_hi);
 }
 
+/* The same idle workgroups also pull the last VT_L2_ROWS gate|up rows of every wave of their XCD
+ * into its L2; those rows are multiplied two phases later and then come from the L2 instead of
+ * HBM, which is idle now. */
+#ifndef VT_L2_ROWS
+#define VT_L2_ROWS 2
+#endif
+
+__device__ __forceinline__ void vt_w13_l2_prefetch(const vt_layer_dev &L) {
+    const int G = (int)gridDim.x, wg = (int)blockIdx.x, nw = (int)(blockDim.x >> 6);
+    if ((G & 7) || wg < VT_HEADS || vt_wave() == 0) return;
+    const int per_x = G >> 3, idle0 = VT_HEADS >> 3;
+    const int me = (((wg >> 3) - idle0) * (nw - 1) + vt_wave() - 1) * VT_WAVE + vt_lane();
+    const int n_lanes = (per_x - idle0) * (nw - 1) * VT_WAVE;
+    int per_wg = (2 * VT_FFN + G - 1) / G;
+    per_wg = (per_wg + 1) / 2 * 2;
+    const int per_wave = (per_wg + nw - 1) / nw;
+    const int lines_per_row = VT_DIM * 2 / 128;
+    const int total = per_x * nw * VT_L2_ROWS * lines_per_row;
+    unsigned acc = 0u;
+    for (int g = me; g < total; g += n_lanes) {
+        const int line = g % lines_per_row, t = g / lines_per_row;
+        const int rr = t % VT_L2_ROWS, wv = (t / VT_L2_ROWS) % nw, i = t / (VT_L2_ROWS * nw);
+        const int row = ((wg & 7) + 8 * i) * per_wg + wv * per_wave + per_wave - VT_L2_ROWS + rr;
+        if (row < 2 * VT_FFN) acc ^= *reinterpret_cast<const unsigned *>(L.w13 + (size_t)row * VT_DIM + line * 64);
+    }
+    asm volatile("" ::"v"(acc));
+}
+
 template <class AR = vt_nothing>
 __device__ __forceinline__ void vt_w13_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
                                             const vt_step_args &a, float *lds, AR after_run = AR()) {
