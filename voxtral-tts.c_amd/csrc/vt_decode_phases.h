@@ -583,6 +583,9 @@ __device__ __forceinline__ void vt_w13_prefetch(u32x4 (&ring)[VT_RING], const vt
 #ifndef VT_L2_ROWS
 #define VT_L2_ROWS 2
 #endif
+#ifndef VT_L2_SKIP
+#define VT_L2_SKIP 24          /* lines of the first prefetched row that are left out: 1.5 rows fit the L2 as well as 2 */
+#endif
 
 __device__ __forceinline__ void vt_w13_l2_prefetch(const vt_layer_dev &L) {
     const int G = (int)gridDim.x, wg = (int)blockIdx.x, nw = (int)(blockDim.x >> 6);
@@ -600,7 +603,8 @@ __device__ __forceinline__ void vt_w13_l2_prefetch(const vt_layer_dev &L) {
         const int line = g % lines_per_row, t = g / lines_per_row;
         const int rr = t % VT_L2_ROWS, wv = (t / VT_L2_ROWS) % nw, i = t / (VT_L2_ROWS * nw);
         const int row = ((wg & 7) + 8 * i) * per_wg + wv * per_wave + per_wave - VT_L2_ROWS + rr;
-        if (row < 2 * VT_FFN) acc ^= *reinterpret_cast<const unsigned *>(L.w13 + (size_t)row * VT_DIM + line * 64);
+        if (row < 2 * VT_FFN && !(rr == 0 && line < VT_L2_SKIP))
+            acc ^= *reinterpret_cast<const unsigned *>(L.w13 + (size_t)row * VT_DIM + line * 64);
     }
     asm volatile("" ::"v"(acc));
 }
