@@ -142,6 +142,12 @@ def test_incomplete_layer_is_an_error(tmp_path):
         save_file(t, str(path))
         assert hip.lib.tts_hip_load_safetensors(str(path).encode()) == -1
         assert hip.pkg.ctx().dec_layers_uploaded == 0
+        # an optional tensor of the wrong size is an error too, not "absent"
+        t = {"acoustic_transformer.input_projection.weight": torch.zeros(S.DIM, S.ACOUSTIC_DIM, dtype=torch.bfloat16),
+             "acoustic_transformer.semantic_codebook_output.bias": torch.zeros(17)}
+        save_file(t, str(path))
+        assert hip.lib.tts_hip_load_safetensors(str(path).encode()) == -1
+        assert b"bias" in hip.lib.tts_hip_last_error() or b"incomplete" in hip.lib.tts_hip_last_error()
     finally:
         hip.close()
 

@@ -211,7 +211,11 @@ static const uint16_t *st_bf16(const st_file *f, const char *name, long long ele
 /* f32 copy (caller frees) of a bf16, f16 or f32 tensor of `elems` elements */
 static float *st_f32(const st_file *f, const char *name, long long elems) {
     const st_tensor *t = st_find(f, name);
-    if (!t || st_count(t) != elems) return NULL;
+    if (!t) return NULL;
+    if (st_count(t) != elems) {                   /* present but of another size: an error, not "absent" */
+        vt_set_error("safetensors: %s has %lld elements, expected %lld", name, st_count(t), elems);
+        return NULL;
+    }
     float *out = (float *)malloc(sizeof(float) * (size_t)elems);
     if (!out) return NULL;
     const unsigned char *src = f->map + f->data0 + t->begin;
@@ -376,6 +380,7 @@ extern "C" int tts_hip_load_safetensors(const char *path) {
     st_file f;
     if (st_open(&f, path)) return -1;
     int mask = 0, rc = 0;
+    const int errs_at_start = g_vt.error_count;
     float *tofree[2 * (TTS_HIP_DEC_LAYERS + TTS_HIP_AC_LAYERS) + 8];
     int nfree = 0;
 
@@ -455,5 +460,8 @@ extern "C" int tts_hip_load_safetensors(const char *path) {
     }
     for (int i = 0; i < nfree; i++) free(tofree[i]);
     st_close(&f);
+    /* a tensor that is present under a known name but has the wrong size or type fails the load,
+     * also where the tensor is optional */
+    if (!rc && g_vt.error_count != errs_at_start) rc = -1;
     return rc ? -1 : mask;
 }
