@@ -186,3 +186,31 @@ def test_barrier_budget_exhausted_is_reported_and_recoverable():
     finally:
         hip.lib.tts_hip_set_barrier_timeout(0)
         hip.close()
+
+
+def test_second_utterance_overwrites_the_cache_rows_of_the_first():
+    """The cache rows of an utterance are read with ordinary (cached) loads, and a second utterance
+    in the same session rewrites rows 0.. with other values: what the attention then reads must be
+    the new rows, also where an L2 still holds the old ones.  Modes 0 and 1, positions that take the
+    per-head attention path."""
+    n_layers, steps = 3, 40
+    layers = [S.Layer(1), S.Layer(2), S.Layer(3)]
+    ones = np.ones(S.DIM, np.float32)
+    hip = H.Hip(kv_max=64)
+    try:
+        hip.upload_decoder(layers, ones, n_layers)
+        for mode in (0, 1):
+            hip.lib.tts_hip_set_decode_mode(mode)
+            for utt, seed in enumerate((100, 200, 300)):
+                orc = cases.OracleBackend(threads=16)
+                orc.llm_open(layers, ones, 64, n_layers=n_layers)
+                hip.pos = 0
+                e = S.f32_normal(S.DIM, seed + mode)
+                for s in range(steps):
+                    ref_h = orc.llm_forward(e)
+                    got_h = hip.llm_forward(e)
+                    assert_close(ref_h, got_h, f"mode {mode} utterance {utt} step {s}")
+                    e = ref_h.copy()
+    finally:
+        hip.lib.tts_hip_set_decode_mode(0)
+        hip.close()
