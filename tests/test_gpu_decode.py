@@ -214,3 +214,45 @@ def test_second_utterance_overwrites_the_cache_rows_of_the_first():
     finally:
         hip.lib.tts_hip_set_decode_mode(0)
         hip.close()
+
+
+def test_backbone_is_the_leading_run_of_complete_layers():
+    """Layers may be uploaded one at a time and in any order; the step runs over the leading
+    layers that are complete, an upload that fails takes its layer out again, and a step without
+    a first layer is an error instead of a launch on missing weights."""
+    import ctypes as C
+    layers = [S.Layer(1), S.Layer(2)]
+    ones = np.ones(S.DIM, np.float32)
+    e = S.f32_normal(S.DIM, 5)
+    hip = H.Hip(kv_max=16)
+    try:
+        lib, pkg = hip.lib, hip.pkg
+        assert lib.tts_hip_upload_llm_norm(ones.ctypes.data) == 0
+        h1 = H.host_layer(pkg, layers[1])
+        assert lib.tts_hip_upload_llm_layer(1, C.byref(h1)) == 0
+        assert pkg.ctx().dec_layers_uploaded == 0              # layer 0 is still missing
+        n0 = lib.tts_hip_error_count()
+        out = np.zeros(S.DIM, np.float32)
+        lib.tts_hip_llm_forward(out.ctypes.data, e.ctypes.data, 0)
+        assert lib.tts_hip_error_count() == n0 + 1 and b"no weights" in lib.tts_hip_last_error()
+        h0 = H.host_layer(pkg, layers[0])
+        assert lib.tts_hip_upload_llm_layer(0, C.byref(h0)) == 0
+        assert pkg.ctx().dec_layers_uploaded == 2
+
+        orc = cases.OracleBackend(threads=8)
+        orc.llm_open(layers, ones, 16, n_layers=2)
+        hip.err0 = lib.tts_hip_error_count()
+        assert_close(orc.llm_forward(e), hip.llm_forward(e), "two layers uploaded one by one")
+
+        # a layer with a missing tensor is refused and the backbone ends in front of it
+        broken = H.host_layer(pkg, layers[1])
+        broken.w2_bf16 = None
+        assert lib.tts_hip_upload_llm_layer(1, C.byref(broken)) == -1
+        assert pkg.ctx().dec_layers_uploaded == 1
+        orc1 = cases.OracleBackend(threads=8)
+        orc1.llm_open(layers[:1], ones, 16, n_layers=1)
+        hip.err0 = lib.tts_hip_error_count()
+        hip.pos = 0
+        assert_close(orc1.llm_forward(e), hip.llm_forward(e), "one layer left")
+    finally:
+        hip.close()

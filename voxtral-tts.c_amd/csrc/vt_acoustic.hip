@@ -748,8 +748,11 @@ extern "C" int tts_hip_upload_audio_embeddings(const uint16_t *emb_bf16, int tot
     if (!g_vt.initialized) { vt_set_error("tts_hip_upload_audio_embeddings: backend not initialised"); return -1; }
     if (!emb_bf16 || !offsets || total_rows < 1) { vt_set_error("tts_hip_upload_audio_embeddings: bad arguments"); return -1; }
     vt_acoustic_dev *ac = &g_vt.ac;
+    VT_TRY(hipStreamSynchronize(g_vt.stream));
     if (ac->audio_emb) (void)hipFree(ac->audio_emb);
     if (ac->audio_offsets) (void)hipFree(ac->audio_offsets);
+    ac->audio_emb = NULL;
+    ac->audio_offsets = NULL;
     ac->audio_rows = 0;
     const size_t bytes = (size_t)total_rows * VT_DIM * 2;
     if (!(ac->audio_emb = (uint16_t *)vt_dev_alloc(bytes))) return -1;

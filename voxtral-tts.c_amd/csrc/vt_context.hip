@@ -75,9 +75,9 @@ static int build_rope_table(int kv_max) {
     return vt_check(e, "rope table upload");
 }
 
-extern "C" int tts_hip_init(int kv_cache_max) {
-    if (g_vt.initialized) return 0;
-    if (kv_cache_max <= 0) { vt_set_error("tts_hip_init: kv_cache_max must be positive"); return -1; }
+static void teardown(void);
+
+static int init_context(int kv_cache_max) {
     int n = 0;
     if (hipGetDeviceCount(&n) != hipSuccess || n == 0) {
         vt_set_error("no HIP device found");
@@ -143,6 +143,16 @@ extern "C" int tts_hip_init(int kv_cache_max) {
     return 0;
 }
 
+extern "C" int tts_hip_init(int kv_cache_max) {
+    if (g_vt.initialized) return 0;
+    if (kv_cache_max <= 0) { vt_set_error("tts_hip_init: kv_cache_max must be positive"); return -1; }
+    if (init_context(kv_cache_max)) {
+        teardown();                 /* a failed init leaves nothing allocated behind */
+        return -1;
+    }
+    return 0;
+}
+
 static void free_layer(vt_layer_dev *l) {
     (void)hipFree((void *)l->wqkv); (void)hipFree((void *)l->wo);
     (void)hipFree((void *)l->w13); (void)hipFree((void *)l->w2);
@@ -150,8 +160,8 @@ static void free_layer(vt_layer_dev *l) {
     memset(l, 0, sizeof *l);
 }
 
-extern "C" void tts_hip_free(void) {
-    if (!g_vt.initialized) return;
+/* Releases whatever the context holds, complete or not; keeps the error count and message. */
+static void teardown(void) {
     (void)hipDeviceSynchronize();
     vt_codec_free();
     for (int i = 0; i < TTS_HIP_DEC_LAYERS; i++) free_layer(&g_vt.h_layers[i]);
@@ -167,13 +177,21 @@ extern "C" void tts_hip_free(void) {
     for (size_t i = 0; i < sizeof ptrs / sizeof ptrs[0]; i++)
         if (ptrs[i]) (void)hipFree(ptrs[i]);
     if (g_vt.h_pin) (void)hipHostFree(g_vt.h_pin);
-    (void)hipEventDestroy(g_vt.ev0);
-    (void)hipEventDestroy(g_vt.ev1);
-    (void)hipStreamDestroy(g_vt.stream);
-    int errs = g_vt.error_count;
+    if (g_vt.ev0) (void)hipEventDestroy(g_vt.ev0);
+    if (g_vt.ev1) (void)hipEventDestroy(g_vt.ev1);
+    if (g_vt.stream) (void)hipStreamDestroy(g_vt.stream);
+    const int errs = g_vt.error_count;
+    char msg[sizeof g_vt.last_error];
+    memcpy(msg, g_vt.last_error, sizeof msg);
     memset(&g_vt, 0, sizeof g_vt);
     g_vt.error_count = errs;
+    memcpy(g_vt.last_error, msg, sizeof msg);
     memset(&g_hip, 0, sizeof g_hip);
+}
+
+extern "C" void tts_hip_free(void) {
+    if (!g_vt.initialized) return;
+    teardown();
 }
 
 extern "C" int tts_hip_available(void) { return g_vt.initialized; }
@@ -199,11 +217,13 @@ static int upload_layer(vt_layer_dev *dst, const tts_hip_host_layer_t *s) {
     }
     free_layer(dst);
     const size_t row = (size_t)VT_DIM * 2;
+    /* every allocation lands in `dst` at once, so that a failure half way leaks nothing: the next
+     * upload of this layer, or the teardown, frees it */
     uint16_t *wqkv = (uint16_t *)vt_dev_alloc((size_t)VT_QKV_DIM * row);
-    uint16_t *w13 = (uint16_t *)vt_dev_alloc((size_t)2 * VT_FFN * row);
-    if (!wqkv || !w13) return -1;
     dst->wqkv = wqkv;
+    uint16_t *w13 = (uint16_t *)vt_dev_alloc((size_t)2 * VT_FFN * row);
     dst->w13 = w13;
+    if (!wqkv || !w13) return -1;
     VT_TRY(hipMemcpy(wqkv, s->wq_bf16, (size_t)VT_Q_DIM * row, hipMemcpyDefault));
     VT_TRY(hipMemcpy(wqkv + (size_t)VT_Q_DIM * VT_DIM, s->wk_bf16, (size_t)VT_KV_DIM * row, hipMemcpyDefault));
     VT_TRY(hipMemcpy(wqkv + (size_t)(VT_Q_DIM + VT_KV_DIM) * VT_DIM, s->wv_bf16, (size_t)VT_KV_DIM * row,
@@ -215,6 +235,21 @@ static int upload_layer(vt_layer_dev *dst, const tts_hip_host_layer_t *s) {
     if (!(dst->attn_norm = (float *)upload(s->attention_norm, sizeof(float) * VT_DIM))) return -1;
     if (!(dst->ffn_norm = (float *)upload(s->ffn_norm, sizeof(float) * VT_DIM))) return -1;
     return 0;
+}
+
+static int layer_complete(const vt_layer_dev *l) {
+    return l->wqkv && l->wo && l->w13 && l->w2 && l->attn_norm && l->ffn_norm;
+}
+
+/* The backbone runs over the leading layers that are completely uploaded; the device's copy of
+ * the layer table follows the host's after every change, so that it never names freed memory. */
+static int publish_dec_layers(void) {
+    int n = 0;
+    while (n < TTS_HIP_DEC_LAYERS && layer_complete(&g_vt.h_layers[n])) n++;
+    g_vt.n_dec_layers = n;
+    g_hip.dec_layers_uploaded = n;
+    return vt_check(hipMemcpy(g_vt.d_layers, g_vt.h_layers, sizeof g_vt.h_layers, hipMemcpyHostToDevice),
+                    "layer table upload");
 }
 
 static int need_init(const char *who) {
@@ -229,11 +264,11 @@ extern "C" int tts_hip_upload_llm_layer(int layer, const tts_hip_host_layer_t *s
         vt_set_error("tts_hip_upload_llm_layer: bad layer index %d", layer);
         return -1;
     }
-    if (upload_layer(&g_vt.h_layers[layer], src)) return -1;
-    VT_TRY(hipMemcpy(g_vt.d_layers, g_vt.h_layers, sizeof g_vt.h_layers, hipMemcpyHostToDevice));
-    if (layer + 1 > g_vt.n_dec_layers) g_vt.n_dec_layers = layer + 1;
-    g_hip.dec_layers_uploaded = g_vt.n_dec_layers;
-    return 0;
+    (void)hipStreamSynchronize(g_vt.stream);
+    const int bad = upload_layer(&g_vt.h_layers[layer], src);
+    if (bad) free_layer(&g_vt.h_layers[layer]);          /* incomplete: the backbone ends in front of it */
+    if (publish_dec_layers()) return -1;
+    return bad ? -1 : 0;
 }
 
 extern "C" int tts_hip_upload_llm_norm(const float *norm) {
@@ -257,16 +292,19 @@ extern "C" int tts_hip_upload_llm_weights_n(void *decoder_ptr, int n_layers) {
     }
     if (!dec->norm) { vt_set_error("tts_hip_upload_llm_weights: NULL final norm"); return -1; }
     if (tts_hip_upload_llm_norm(dec->norm)) return -1;
+    (void)hipStreamSynchronize(g_vt.stream);
     g_vt.n_dec_layers = 0;
-    for (int i = 0; i < n_layers; i++) {
-        if (upload_layer(&g_vt.h_layers[i], &dec->layers[i])) {
+    for (int i = 0; i < TTS_HIP_DEC_LAYERS; i++) {
+        if (i < n_layers && upload_layer(&g_vt.h_layers[i], &dec->layers[i])) {
             fprintf(stderr, "tts_hip: failed to upload LLM layer %d\n", i);
+            free_layer(&g_vt.h_layers[i]);
+            (void)publish_dec_layers();
             return -1;
         }
+        if (i >= n_layers) free_layer(&g_vt.h_layers[i]);    /* a shorter backbone than before */
     }
-    VT_TRY(hipMemcpy(g_vt.d_layers, g_vt.h_layers, sizeof g_vt.h_layers, hipMemcpyHostToDevice));
-    g_vt.n_dec_layers = n_layers;
-    g_hip.dec_layers_uploaded = n_layers;
+    if (publish_dec_layers()) return -1;
+    if (g_vt.n_dec_layers != n_layers) { vt_set_error("tts_hip_upload_llm_weights: internal layer count"); return -1; }
     return 0;
 }
 
@@ -279,11 +317,16 @@ extern "C" int tts_hip_upload_acoustic_weights(void *acoustic_ptr) {
     tts_hip_host_acoustic_t *ac = (tts_hip_host_acoustic_t *)acoustic_ptr;
     if (!ac) { vt_set_error("tts_hip_upload_acoustic_weights: NULL"); return -1; }
     vt_acoustic_dev *d = &g_vt.ac;
-    void *old[] = {d->input_proj, d->time_proj, d->llm_proj, d->semantic_out, d->acoustic_out,
-                   d->semantic_bias, d->norm, d->time_inv_freq, d->time_tok};
-    for (size_t i = 0; i < sizeof old / sizeof old[0]; i++) if (old[i]) (void)hipFree(old[i]);
+    (void)hipStreamSynchronize(g_vt.stream);
+    void **old[] = {(void **)&d->input_proj, (void **)&d->time_proj, (void **)&d->llm_proj,
+                    (void **)&d->semantic_out, (void **)&d->acoustic_out, (void **)&d->semantic_bias,
+                    (void **)&d->norm, (void **)&d->time_inv_freq, (void **)&d->time_tok};
+    for (size_t i = 0; i < sizeof old / sizeof old[0]; i++) {
+        if (*old[i]) (void)hipFree(*old[i]);
+        *old[i] = NULL;              /* a failure below must not leave a freed pointer for the teardown */
+    }
     g_vt.ac_uploaded = 0;
-    d->semantic_bias = NULL;
+    g_hip.ac_layers_uploaded = 0;
     d->time_tok_ready = 0;
     if (!(d->time_tok = (float *)vt_dev_alloc(sizeof(float) * 8 * VT_DIM))) return -1;
     if (!(d->input_proj = (uint16_t *)upload(ac->input_proj_bf16, (size_t)VT_DIM * VT_AC_DIM_IN * 2))) return -1;
