@@ -500,12 +500,88 @@ def bench_frame(args):
     print(json.dumps(out))
 
 
+MATVEC_SHAPES = ((9216, 3072, "FFN up/gate"), (3072, 9216, "FFN down"), (131072, 3072, "LM-head sized"))
+
+
+def bench_matvec(args):
+    """The single bf16 matvec of configs[0]: y = W x, W bf16 ~N(0,0.02), x f32 ~N(0,1), the three
+    shapes of the reference's CPU kernel.  A step is one product; launches rotate through copies of
+    the two small matrices (8 x 56.6 MB) so that every one streams from HBM, not the memory-side cache."""
+    import cases
+    K, W = args.steps, args.warmup
+    hip = H.Hip(kv_max=8)
+    lib = hip.lib
+    cpu_lib = cases.RefBackend() if S.have_ref() else cases.OracleBackend(threads=1)
+    kind = "reference" if S.have_ref() else "port"
+    per_shape, t_gen, t_up = {}, 0.0, 0.0
+    cpu_ms, parity = {}, {}
+    for n, k, what in MATVEC_SHAPES:
+        t0 = time.time()
+        Wm = S.bf16_normal((n, k), 1000 + n % 97 + k)
+        x = S.f32_normal((1, k), 42)
+        t_gen += time.time() - t0
+        nbytes = 2 * n * k + 4 * k + 4 * n
+        copies = 8 if 2 * n * k < (512 << 20) else 1
+        t0 = time.time()
+        d_W = H.DevBuf(lib, copies * 2 * n * k)
+        for c in range(copies):
+            lib.tts_hip_to_device(d_W.at(c * 2 * n * k), Wm.ctypes.data, 2 * n * k)
+        d_x = H.DevBuf.from_numpy(lib, x)
+        d_y = H.DevBuf(lib, 4 * n)
+        t_up += time.time() - t0
+        ms = lib.tts_hip_bench_matvec(d_y.ptr, d_x.ptr, d_W.ptr, n * k, copies, k, n, max(K, copies))
+        hip.check()
+        got = d_y.to_numpy(np.float32, (1, n))
+        name = f"{n}x{k}"
+        per_shape[name] = {"what": what, "us": round(ms * 1e3, 2), "bytes": nbytes,
+                           "gbps": round(nbytes / ms / 1e6, 1), "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                           "copies": copies}
+        if args.cpu_seconds > 0:
+            reps = 3 if n * k < (1 << 28) else 1
+            t0 = time.time()
+            for _ in range(reps):
+                ref = cpu_lib.linear(x, Wm, None, 1)
+            cpu_ms[name] = round((time.time() - t0) / reps * 1e3, 1)
+            mx, l2 = S.rel_errors(ref, got)
+            parity[name] = {"max_abs_over_rms": float(f"{mx:.3g}"), "l2_rel": float(f"{l2:.3g}")}
+            assert mx < 1e-3 and l2 < 1e-3, (name, mx, l2)
+        for b in (d_W, d_x, d_y):
+            b.free()
+    big = per_shape["131072x3072"]
+    out = {
+        "metric": "bf16 matvec achieved HBM GB/s (131072x3072)",
+        "value": big["gbps"], "unit": "GB/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(big["us"] / 1e3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "single bf16 matvec y = W x, batch 1, fp32 accumulate (BASELINE.json configs[0]): "
+                               "9216x3072, 3072x9216 and 131072x3072",
+                   "weights": "bf16 N(0,0.02) seeded, truncated", "activations": "f32 N(0,1)",
+                   "timed": "events on the library's stream, operands resident in HBM"},
+        "per_shape": per_shape,
+        "roofline": {"kernel": "vt_matvec_kernel (131072x3072)", "bound": "hbm", "achieved": big["gbps"],
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": big["frac"], "traffic": measured_traffic("matvec"),
+                     "bytes_per_launch": big["bytes"], "ms_per_launch": round(big["us"] / 1e3, 5)},
+        "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
+        "cpu_baseline": None,
+    }
+    if cpu_ms:
+        name = "131072x3072"
+        out["cpu_baseline"] = {"value": round(per_shape[name]["bytes"] / cpu_ms[name] / 1e6, 2), "unit": "GB/s",
+                               "cores": 1, "kind": kind, "ms": cpu_ms,
+                               "sample": "the same three products through the reference's tts_linear_bf16 "
+                                         "(bf16_matvec_fused), one thread, 3 / 3 / 1 repetitions"}
+        out["parity"] = parity
+    hip.close()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=("decode", "prefill", "acoustic", "frame", "codec"), default="decode",
+    ap.add_argument("--workload", choices=("decode", "prefill", "acoustic", "frame", "codec", "matvec"), default="decode",
                     help="decode = the headline metric; prefill / acoustic = the other two configurations")
     ap.add_argument("--mode", type=int, default=0, help="0 persistent kernel, 1 per-phase kernels, 2 streaming kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
@@ -527,6 +603,8 @@ def main():
         return bench_codec(args)
     if args.workload == "frame":
         return bench_frame(args)
+    if args.workload == "matvec":
+        return bench_matvec(args)
     K, W = args.steps, args.warmup
     workers = min(16, os.cpu_count() or 8)
 

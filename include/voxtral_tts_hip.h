@@ -284,6 +284,13 @@ float tts_hip_timer_stop_ms(void);
  * product at 1600 rows with the q|k|v, output, gate|up and down matrices, 24 = the whole codec
  * decoder on 200 frames (codec weights uploaded).  Negative on error. */
 float tts_hip_bench_kernel(int which, int iters);
+/* Average duration in ms of one single-row product y[out_dim] = W[out_dim, in_dim] x (the kernel
+ * behind tts_hip_linear_bf16 with seq_len 1), timed with events on the internal stream over
+ * `iters` launches.  Launch i reads copy i % n_copies of W, `copy_stride` elements apart, so that
+ * a matrix smaller than the memory-side cache is streamed from HBM every time.  Device pointers.
+ * Negative on error. */
+float tts_hip_bench_matvec(float *d_y, const float *d_x, const uint16_t *d_W, size_t copy_stride,
+                           int n_copies, int in_dim, int out_dim, int iters);
 
 #ifdef __cplusplus
 }

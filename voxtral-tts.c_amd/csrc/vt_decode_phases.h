@@ -198,12 +198,48 @@ __device__ __forceinline__ void vt_ring_prefetch(u32x4 (&ring)[VT_RING], const u
     }
 }
 
-/* Consume the wave's rows: y_lds[part * wg_nrows + local_row] = partial dot. */
+/* Consume the wave's rows: y_lds[part * wg_nrows + local_row] = partial dot.
+ *
+ * The compiler counts outstanding loads statically: behind a load that is issued under a
+ * condition it has to wait as if that load were not there, i.e. for everything.  With the row
+ * count as a template parameter the loop below unrolls into straight-line code in which every
+ * request is unconditional, and each row then waits for exactly the loads older than its own:
+ * the D - 1 younger rows stay in flight while it is multiplied.  The scheduling barriers keep a
+ * row's requests where they are written, behind the last use of the registers they overwrite. */
+template <int NK, int D, int NR>
+__device__ __forceinline__ void vt_ring_run_fixed(u32x4 (&ring)[VT_RING], const uint16_t *W,
+                                                  int row_len, const vt_rows &r,
+                                                  const f32x4 (&xa)[NK], const f32x4 (&xb)[NK],
+                                                  float *y_lds) {
+    const uint16_t *base = W + (size_t)r.r0 * row_len + r.kofs + vt_lane() * 8;
+    float *y = y_lds + r.part * r.wg_nrows + (r.r0 - r.wg_row0);
+#pragma unroll
+    for (int row = 0; row < NR; row++) {
+        const int j = row % D;
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int c = 0; c < NK; c += 2) {
+            a0 = vt_dot8(ring[j * NK + c], xa[c], xb[c], a0);
+            if (c + 1 < NK) a1 = vt_dot8(ring[j * NK + c + 1], xa[c + 1], xb[c + 1], a1);
+        }
+        if (row + D < NR) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int c = 0; c < NK; c++)
+                ring[j * NK + c] = vt_ldw(base + (size_t)(row + D) * row_len + c * 512);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const float s = vt_wave_sum(a0 + a1);
+        if (vt_lane() == 0) y[row] = s;
+    }
+}
+
+/* Any row count: rows and requests under run-time conditions (see above for what that costs). */
 template <int NK, int D>
-__device__ __forceinline__ void vt_ring_run(u32x4 (&ring)[VT_RING], const uint16_t *W,
-                                            int row_len, const vt_rows &r,
-                                            const f32x4 (&xa)[NK], const f32x4 (&xb)[NK],
-                                            float *y_lds) {
+__device__ __forceinline__ void vt_ring_run_any(u32x4 (&ring)[VT_RING], const uint16_t *W,
+                                                int row_len, const vt_rows &r,
+                                                const f32x4 (&xa)[NK], const f32x4 (&xb)[NK],
+                                                float *y_lds) {
     const uint16_t *base = W + (size_t)r.r0 * row_len + r.kofs + vt_lane() * 8;
     float *y = y_lds + r.part * r.wg_nrows + (r.r0 - r.wg_row0);
     for (int i = 0; i < r.nr; i += D) {
@@ -229,6 +265,16 @@ __device__ __forceinline__ void vt_ring_run(u32x4 (&ring)[VT_RING], const uint16
     }
 }
 
+/* NR: the row count of a wave on a 256-workgroup grid, where the straight-line version runs. */
+template <int NK, int D, int NR>
+__device__ __forceinline__ void vt_ring_run(u32x4 (&ring)[VT_RING], const uint16_t *W,
+                                            int row_len, const vt_rows &r,
+                                            const f32x4 (&xa)[NK], const f32x4 (&xb)[NK],
+                                            float *y_lds) {
+    if (r.nr == NR) vt_ring_run_fixed<NK, D, NR>(ring, W, row_len, r, xa, xb, y_lds);
+    else vt_ring_run_any<NK, D>(ring, W, row_len, r, xa, xb, y_lds);
+}
+
 /* ---- phase 1: RMSNorm + [wq;wk;wv] + RoPE + cache append ------------------ */
 
 __device__ __forceinline__ vt_rows vt_qkv_rows() { return vt_split_rows<1>(VT_QKV_DIM, 2, 0); }
@@ -251,7 +297,7 @@ __device__ __forceinline__ void vt_qkv_body(u32x4 (&ring)[VT_RING], const vt_lay
     vt_stage(lds, x_in, VT_DIM);
     f32x4 xa[6], xb[6];
     vt_rmsnorm_slice(xa, xb, lds, L.attn_norm);
-    vt_ring_run<6, 3>(ring, L.wqkv, VT_DIM, r, xa, xb, lds_y);
+    vt_ring_run<6, 3, 3>(ring, L.wqkv, VT_DIM, r, xa, xb, lds_y);
     after_run();
     __syncthreads();
     /* RoPE on adjacent pairs (voxtral_tts_kernels.c:616-634), then q to its
@@ -557,7 +603,7 @@ __device__ __forceinline__ void vt_wo_body(u32x4 (&ring)[VT_RING], const vt_laye
     /* the residual value of this thread's row, requested before any bulk load of the next phase */
     const int tr = (int)threadIdx.x < r.wg_nrows ? (int)threadIdx.x : 0;
     const float prev = vt_ldc(x_in + r.wg_row0 + tr);
-    vt_ring_run<4, 4>(ring, L.wo, VT_Q_DIM, r, xa, xb, lds_y);
+    vt_ring_run<4, 4, 3>(ring, L.wo, VT_Q_DIM, r, xa, xb, lds_y);
     after_run();
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows; t += (int)blockDim.x) {
@@ -617,7 +663,7 @@ __device__ __forceinline__ void vt_w13_body(u32x4 (&ring)[VT_RING], const vt_lay
     vt_stage(lds, a.x, VT_DIM);
     f32x4 xa[6], xb[6];
     vt_rmsnorm_slice(xa, xb, lds, L.ffn_norm);
-    vt_ring_run<6, 3>(ring, L.w13, VT_DIM, r, xa, xb, lds_y);
+    vt_ring_run<6, 3, 9>(ring, L.w13, VT_DIM, r, xa, xb, lds_y);
     after_run();
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows / 2; t += (int)blockDim.x) {
@@ -646,7 +692,7 @@ __device__ __forceinline__ void vt_w2_body(u32x4 (&ring)[VT_RING], const vt_laye
     vt_slice_lds<9>(xa, xb, lds, r.kofs);
     const int tr = (int)threadIdx.x < r.wg_nrows ? (int)threadIdx.x : 0;
     const float prev = vt_ldc(a.x + r.wg_row0 + tr);
-    vt_ring_run<9, 2>(ring, L.w2, VT_FFN, r, xa, xb, lds_y);
+    vt_ring_run<9, 2, 3>(ring, L.w2, VT_FFN, r, xa, xb, lds_y);
     after_run();
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows; t += (int)blockDim.x) {

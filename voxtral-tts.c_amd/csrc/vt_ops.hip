@@ -54,8 +54,130 @@ vt_linear_kernel(float *y, const float *x, const uint16_t *W, const float *bias,
     }
 }
 
+/* Single-row product y = W x as one stream (the decode GEMV of bf16_matvec_fused,
+ * voxtral_tts_kernels.c:152-185).  A workgroup owns `rows_per_wg` consecutive rows, i.e. one
+ * contiguous piece of W, and cuts it into 8 equal runs of 1 KB chunks (512 weights: 16 bytes per
+ * lane), one per wave, wherever the row boundaries fall: every wave streams the same number of
+ * bytes whatever the shape.  A wave keeps MV_RING chunks requested ahead (non-temporal 16-byte
+ * loads, the first ones before x is even staged), multiplies each against the matching slice of
+ * x in LDS, and leaves one partial sum per row it touched in part[row][wave]; the partials of a
+ * row are added in wave order, so the result does not depend on timing.  x sits in LDS as
+ * [chunk][half][lane][4] so that the two 16-byte reads of a lane are contiguous over the wave. */
+#define MV_RING 16
+#define MV_THREADS 512
+#define MV_MAX_ROWS 512          /* rows per workgroup: part[] is MV_MAX_ROWS x 8 floats */
+
+__global__ void __launch_bounds__(MV_THREADS)
+vt_matvec_kernel(float *y, const float *x, const uint16_t *W, const float *bias, int in_dim, int out_dim,
+                 int rows_per_wg) {
+    extern __shared__ __attribute__((aligned(16))) float mv_lds[];
+    float *xs = mv_lds, *part = mv_lds + in_dim;
+    const int tid = (int)threadIdx.x, lane = vt_lane(), nw = (int)(blockDim.x >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(vt_wave());      /* uniform: the loop bounds below are scalars */
+    const int row0 = (int)blockIdx.x * rows_per_wg;
+    const int rows = min(rows_per_wg, out_dim - row0);
+    if (rows <= 0) return;
+    const int cpr = in_dim >> 9;                                     /* chunks per row */
+    const int n_wg = rows * cpr;
+    const int c_lo = (int)((long long)n_wg * wave / nw), c_hi = (int)((long long)n_wg * (wave + 1) / nw);
+    const int n = c_hi - c_lo;
+    const uint16_t *base = W + (size_t)row0 * in_dim + (size_t)c_lo * 512 + lane * 8;
+    u32x4 ring[MV_RING];
+    const bool steady = n >= 2 * MV_RING;        /* then the first round is requested without conditions, too */
+    if (steady) {
+#pragma unroll
+        for (int i = 0; i < MV_RING; i++) ring[i] = vt_ldw(base + (size_t)i * 512);
+    } else {
+#pragma unroll
+        for (int i = 0; i < MV_RING; i++)
+            if (i < n) ring[i] = vt_ldw(base + (size_t)i * 512);
+    }
+    for (int g = tid; g < in_dim / 4; g += (int)blockDim.x) {
+        const int kc = g >> 7, within = g & 127;
+        *reinterpret_cast<f32x4 *>(xs + kc * 512 + (within & 1) * 256 + (within >> 1) * 4) =
+            *reinterpret_cast<const f32x4 *>(x + 4 * g);
+    }
+    for (int i = tid; i < rows * nw; i += (int)blockDim.x) part[i] = 0.f;
+    __syncthreads();
+    int r = c_lo / cpr, kc = c_lo % cpr;
+    float acc = 0.f;
+    const int dummy = rows * nw + tid;                 /* behind the partial sums */
+    /* steady state: every slot is requested again as soon as it has been multiplied, without a
+     * condition, so that the wait for slot j + 1 lets the 15 younger requests stay in flight */
+    int c0 = 0;
+    for (; c0 + 2 * MV_RING <= n; c0 += MV_RING) {
+#pragma unroll
+        for (int j = 0; j < MV_RING; j++) {
+            const float *xp = xs + kc * 512 + lane * 4;
+            acc = vt_dot8(ring[j], *reinterpret_cast<const f32x4 *>(xp), *reinterpret_cast<const f32x4 *>(xp + 256), acc);
+            /* the request stays behind the last use of the registers it overwrites: hoisted, it would
+             * land in other registers and be copied back at the end of the round, behind a wait for all */
+            __builtin_amdgcn_sched_barrier(0);
+            ring[j] = vt_ldw(base + (size_t)(c0 + j + MV_RING) * 512);
+            __builtin_amdgcn_sched_barrier(0);
+            /* no branch in this loop (behind one the compiler waits for every outstanding load):
+             * the row sum is formed after every chunk and stored to a dummy slot unless the row ends */
+            const bool end = ++kc == cpr;
+            const float sum = vt_wave_sum(acc);
+            part[lane == 0 && end ? r * nw + wave : dummy] = sum;
+            acc = end ? 0.f : acc;
+            r += end ? 1 : 0;
+            kc = end ? 0 : kc;
+        }
+    }
+    /* the last one or two rounds: requests only while chunks are left */
+    for (; c0 < n; c0 += MV_RING) {
+#pragma unroll
+        for (int j = 0; j < MV_RING; j++) {
+            const int c = c0 + j;
+            if (c < n) {
+                const u32x4 w = ring[j];
+                if (c + MV_RING < n) ring[j] = vt_ldw(base + (size_t)(c + MV_RING) * 512);
+                const float *xp = xs + kc * 512 + lane * 4;
+                acc = vt_dot8(w, *reinterpret_cast<const f32x4 *>(xp), *reinterpret_cast<const f32x4 *>(xp + 256), acc);
+                if (++kc == cpr || c == n - 1) {
+                    const float sum = vt_wave_sum(acc);
+                    if (lane == 0) part[r * nw + wave] = sum;
+                    r++;
+                    kc = 0;
+                    acc = 0.f;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (int i = tid; i < rows; i += (int)blockDim.x) {
+        float sum = 0.f;
+        for (int w = 0; w < nw; w++) sum = __fadd_rn(sum, part[i * nw + w]);
+        y[row0 + i] = bias ? __fadd_rn(bias[row0 + i], sum) : sum;
+    }
+}
+
+/* Shapes the stream kernel takes: whole 1 KB chunks per row, 16-byte aligned operands, x and the
+ * partial sums within the 64 KB of LDS a workgroup gets without asking. */
+static int matvec_launch(float *d_y, const float *d_x, const uint16_t *d_W, const float *d_bias,
+                         int in_dim, int out_dim) {
+    if (in_dim % 512 != 0 || (((uintptr_t)d_W | (uintptr_t)d_x) & 15)) return 0;
+    /* one workgroup per CU for matrices of a few rounds per wave; up to four (two resident, the
+     * others queued behind them) where a wave would otherwise run more than three rounds of its
+     * ring: measured 6.3 -> 6.7 TB/s on 131072 x 3072, while 9216 x 3072 is fastest with one */
+    const int n_cu = g_vt.n_cu > 0 ? g_vt.n_cu : 256;
+    const long long chunks = (long long)out_dim * (in_dim / 512);
+    long long want = chunks / ((MV_THREADS / 64) * 3 * MV_RING);
+    const int n_wg = (int)(want < n_cu ? n_cu : (want > 4 * n_cu ? 4 * n_cu : want));
+    int rows_per_wg = (out_dim + n_wg - 1) / n_wg;
+    if (rows_per_wg > MV_MAX_ROWS) rows_per_wg = MV_MAX_ROWS;
+    const size_t lds = sizeof(float) * ((size_t)in_dim + (size_t)rows_per_wg * (MV_THREADS / 64) + MV_THREADS);
+    if (lds > 65536) return 0;
+    const int grid = (out_dim + rows_per_wg - 1) / rows_per_wg;
+    hipLaunchKernelGGL(vt_matvec_kernel, dim3(grid), dim3(MV_THREADS), lds, g_vt.stream, d_y, d_x, d_W, d_bias,
+                       in_dim, out_dim, rows_per_wg);
+    return 1;
+}
+
 void vt_launch_linear(float *d_y, const float *d_x, const uint16_t *d_W, const float *d_bias,
                       int seq_len, int in_dim, int out_dim) {
+    if (seq_len == 1 && matvec_launch(d_y, d_x, d_W, d_bias, in_dim, out_dim)) return;
     const int vec_ok = (in_dim % 8 == 0) && (((uintptr_t)d_W | (uintptr_t)d_x) % 16 == 0);
     const dim3 grid((out_dim + 3) / 4), block(256);
     if (seq_len == 1)
@@ -139,6 +261,26 @@ done:
     if (tmp_x) (void)hipFree(tmp_x);
     if (tmp_y) (void)hipFree(tmp_y);
     if (tmp_W) (void)hipFree(tmp_W);
+}
+
+extern "C" float tts_hip_bench_matvec(float *d_y, const float *d_x, const uint16_t *d_W, size_t copy_stride,
+                                      int n_copies, int in_dim, int out_dim, int iters) {
+    if (!g_vt.initialized) { vt_set_error("tts_hip_bench_matvec: backend not initialised"); return -1.f; }
+    if (!d_y || !d_x || !d_W || n_copies < 1 || in_dim < 1 || out_dim < 1 || iters < 1) {
+        vt_set_error("tts_hip_bench_matvec: bad arguments");
+        return -1.f;
+    }
+    for (int i = 0; i < n_copies; i++)                                  /* warm-up: one pass over every copy */
+        vt_launch_linear(d_y, d_x, d_W + (size_t)i * copy_stride, NULL, 1, in_dim, out_dim);
+    if (vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench record")) return -1.f;
+    for (int i = 0; i < iters; i++)
+        vt_launch_linear(d_y, d_x, d_W + (size_t)(i % n_copies) * copy_stride, NULL, 1, in_dim, out_dim);
+    if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench record")) return -1.f;
+    if (vt_check(hipEventSynchronize(g_vt.ev1), "bench sync")) return -1.f;
+    if (vt_check(hipGetLastError(), "bench launch")) return -1.f;
+    float ms = -1.f;
+    if (vt_check(hipEventElapsedTime(&ms, g_vt.ev0, g_vt.ev1), "bench elapsed")) return -1.f;
+    return ms / (float)iters;
 }
 
 /* ---- RMSNorm: one workgroup per row ------------------------------------------ */
