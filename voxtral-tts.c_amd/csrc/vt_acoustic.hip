@@ -288,24 +288,41 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
         if (PH == AC_WO) ac_attention_to_planes(hi, lo, SH::PITCH, ra);
         else ac_rows_to_planes<true>(hi, lo, SH::PITCH, rr, red_ss);
         __syncthreads();
+        /* The request for unit u + G is never issued under a condition of its own: the compiler
+         * counts outstanding loads statically, and behind a conditional request it would make the
+         * product of unit u wait for unit u + G as well (which is what the two register sets are
+         * there to avoid).  The last unit of a workgroup takes the branch without a request. */
+        float *red1 = red + AC_WAVES * AC_ROWS * 16;
         for (;;) {
+            int nx = u + G;
+            if (nx >= n_units) {
+                f32x4 ah = zero4, al = zero4;
+                ac_consume(w0, fa, fl, ah, al);
+                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al);
+                break;
+            }
             {
-                const int nx = u + G;
-                if (nx < n_units) ac_issue<PH>(w1, wbase + nx * unit_stride);
+                ac_issue<PH>(w1, wbase + nx * unit_stride);
+                __builtin_amdgcn_sched_barrier(0);
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w0, fa, fl, ah, al);
                 ac_finish_unit<PH>(a, red, u * AC_RB, ah, al);
                 u = nx;
-                if (u >= n_units) break;
             }
-            {
-                const int nx = u + G;
-                if (nx < n_units) ac_issue<PH>(w0, wbase + nx * unit_stride);
+            nx = u + G;
+            if (nx >= n_units) {
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w1, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red + AC_WAVES * AC_ROWS * 16, u * AC_RB, ah, al);
+                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al);
+                break;
+            }
+            {
+                ac_issue<PH>(w0, wbase + nx * unit_stride);
+                __builtin_amdgcn_sched_barrier(0);
+                f32x4 ah = zero4, al = zero4;
+                ac_consume(w1, fa, fl, ah, al);
+                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al);
                 u = nx;
-                if (u >= n_units) break;
             }
         }
     } else {
