@@ -78,9 +78,9 @@ vt_codec_gemm_kernel(float *__restrict__ C, const float *__restrict__ A, const f
         ap[p] = A + (size_t)am * lda + kbeg + lc;
         wp[p] = W + (size_t)(n0 + p * 32 + lr) * K + kbeg + lc;
     }
-    float4 ra[4], rw[4];
+    f32x4 ra[4], rw[4];       /* clang vectors: HIP's float4 structs in an array end up in LDS, not registers */
 #pragma unroll
-    for (int p = 0; p < 4; p++) { ra[p] = *(const float4 *)ap[p]; rw[p] = *(const float4 *)wp[p]; }
+    for (int p = 0; p < 4; p++) { ra[p] = *(const f32x4 *)ap[p]; rw[p] = *(const f32x4 *)wp[p]; }
 
     cd_f16v acc[2][2];
 #pragma unroll
@@ -95,24 +95,29 @@ vt_codec_gemm_kernel(float *__restrict__ C, const float *__restrict__ A, const f
         __syncthreads();
 #pragma unroll
         for (int p = 0; p < 4; p++) {
-            *(float4 *)&As[(p * 32 + lr) * CG_PITCH + lc] = ra[p];
-            *(float4 *)&Ws[(p * 32 + lr) * CG_PITCH + lc] = rw[p];
+            *(f32x4 *)&As[(p * 32 + lr) * CG_PITCH + lc] = ra[p];
+            *(f32x4 *)&Ws[(p * 32 + lr) * CG_PITCH + lc] = rw[p];
         }
         __syncthreads();
-        if (k0 + CG_BK < kper) {
+        {
+            /* the next K step is requested without a condition (the last step asks for its own
+             * tile again, out of the L2): behind a conditional request the compiler parks the
+             * registers in LDS and waits for the loads before the products instead of after */
+            const int kn = k0 + CG_BK < kper ? k0 + CG_BK : k0;
 #pragma unroll
             for (int p = 0; p < 4; p++) {
-                ra[p] = *(const float4 *)(ap[p] + k0 + CG_BK);
-                rw[p] = *(const float4 *)(wp[p] + k0 + CG_BK);
+                ra[p] = *(const f32x4 *)(ap[p] + kn);
+                rw[p] = *(const f32x4 *)(wp[p] + kn);
             }
+            __builtin_amdgcn_sched_barrier(0);          /* requests first, products behind them */
         }
 #pragma unroll
         for (int kg = 0; kg < CG_BK; kg += 8) {
-            float4 fa[2], fw[2];
+            f32x4 fa[2], fw[2];
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                fa[i] = *(const float4 *)&As[(wm * 64 + i * 32 + fr) * CG_PITCH + kg + fk];
-                fw[i] = *(const float4 *)&Ws[(wn * 64 + i * 32 + fr) * CG_PITCH + kg + fk];
+                fa[i] = *(const f32x4 *)&As[(wm * 64 + i * 32 + fr) * CG_PITCH + kg + fk];
+                fw[i] = *(const f32x4 *)&Ws[(wn * 64 + i * 32 + fr) * CG_PITCH + kg + fk];
             }
 #pragma unroll
             for (int i = 0; i < 2; i++)
