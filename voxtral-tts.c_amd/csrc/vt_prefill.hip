@@ -122,7 +122,11 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
             rv[i] = *reinterpret_cast<const f32x4 *>(Vc + (size_t)kr * VT_KV_DIM + kvh * VT_HEAD_DIM + col);
         }
     };
-    if (pz < ntiles) fetch(pz);
+    /* Every request of the loop below is unconditional (a tile index beyond the last visible one
+     * is clamped: that tile is fetched again, out of the L2, and never stored): behind a
+     * conditional request the compiler waits for all outstanding loads before the next use of
+     * anything loaded, here the query registers, i.e. before the products of every step. */
+    fetch(pz < ntiles ? pz : ntiles - 1);
 
     for (int step = 0; step < nsteps; step++) {
         const int tile = step * NSPLIT + pz;
@@ -137,7 +141,8 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
             }
         }
         __syncthreads();
-        if (tile + NSPLIT < ntiles) fetch(tile + NSPLIT);
+        fetch(tile + NSPLIT < ntiles ? tile + NSPLIT : ntiles - 1);
+        __builtin_amdgcn_sched_barrier(0);               /* requests first, products behind them */
         if (!valid) continue;
 
         /* S^T = K Q^T: reduction step (j, e) pairs dim 32*g + 4*j + e of key and query */
