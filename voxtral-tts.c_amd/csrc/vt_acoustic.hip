@@ -18,9 +18,10 @@
  *   attention (3x3 per head and branch) + output projection + residual
  *   RMSNorm + gate/up + SiLU*up -> h [6, 9216]
  *   down projection + residual
- * A one-workgroup kernel closes a step (final norm, 36-wide output
- * projection of both branches, guided Euler update) and opens the next one
- * (input projection of the new latent, token assembly).
+ * Two small kernels stand between the steps: one closes a step (final norm,
+ * 36-wide output projection of both branches), the other applies the guided
+ * Euler update and opens the next step (input projection of the new latent,
+ * token assembly).
  */
 #include "vt_state.h"
 
@@ -349,121 +350,149 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
     }
 }
 
-/* ---- step boundary: one workgroup ---------------------------------------------- */
+/* ---- step boundary ------------------------------------------------------------------
+ * Two small launches: `back` closes a step (final norm of token 0 of both branches, the 72
+ * dot products of the 36-wide output projection), `front` applies the guided Euler update,
+ * quantises at the end of the frame, and opens the next step (36-term input projection of the
+ * new latent, token assembly).  Both used to be one workgroup, which then pulled the two
+ * 221 KB matrices through a single CU (18 us per step); spread over 5 and 3 workgroups the
+ * same arithmetic, element for element, takes a few microseconds per launch.  The latent is
+ * read from x_in and written to x_out by workgroup 0 only (every workgroup of `front` applies
+ * the update for itself; in place, a late workgroup would apply it twice). */
 
 struct ac_edge_args {
-    const float *tok_in;          /* [6,3072] after the last layer (back part) */
-    float *tok_out;               /* [6,3072] for the next step (front part) */
+    const float *tok_in;          /* [6,3072] after the last layer (back) */
+    float *tok_out;               /* [6,3072] for the next step (front, when do_front) */
     const float *norm;            /* final norm gains */
     const uint16_t *acoustic_out; /* [36,3072] */
     const uint16_t *input_proj;   /* [3072,36] */
     const float *time_tok;        /* [3072] projected time token of the next step */
     const float *llm_tok;         /* [3072] projected LLM token */
-    float *x;                     /* [36] latent, updated in place */
-    float *vel;                   /* [72] cond | uncond velocities (written when do_back) */
+    const float *x_in;            /* [36] latent */
+    float *x_out;                 /* [36] latent after the update (== x_in values without do_euler) */
+    float *vel;                   /* [72] cond | uncond velocities (written by back, read by front) */
     int *codes;                   /* [37] (FSQ codes at 1..36 when do_fsq) */
     float dt;
-    int do_back, do_euler, do_front, do_fsq;
+    int do_euler, do_front, do_fsq;
 };
 
+#define AC_BACK_WGS 5             /* x 16 waves >= 72 dot products */
+#define AC_FRONT_WGS 3            /* x 1024 threads = 3072 token columns */
+
 __global__ void __launch_bounds__(1024)
-vt_ac_edge_kernel(ac_edge_args a) {
+vt_ac_edge_back_kernel(ac_edge_args a) {
     __shared__ float red[2][16];
     __shared__ float s_inv[2];
-    __shared__ float s_vel[2 * VT_AC_DIM_IN];
-    __shared__ float s_x[VT_AC_DIM_IN];
     __shared__ __attribute__((aligned(16))) float s_xn[2][VT_DIM];
     const int t = (int)threadIdx.x, lane = vt_lane(), wave = vt_wave();
-    if (t < VT_AC_DIM_IN) s_x[t] = a.x[t];
-    if (a.do_back) {
-        /* final RMSNorm of token 0 of each branch (rows 0 and 3), then the 36-wide projection
-         * (voxtral_tts_acoustic.c:255-261) */
-        float v[2][3];
+    /* this wave's row of the projection is requested first: it does not depend on the tokens */
+    const int o = (int)blockIdx.x * 16 + wave;
+    const bool mine = o < 2 * VT_AC_DIM_IN;
+    const int ob = mine ? o / VT_AC_DIM_IN : 0, orow = mine ? o % VT_AC_DIM_IN : 0;
+    u32x4 w[VT_DIM / 512];
 #pragma unroll
-        for (int b = 0; b < 2; b++) {
-            float ss = 0.f;
+    for (int i = 0; i < VT_DIM / 512; i++)
+        w[i] = *reinterpret_cast<const u32x4 *>(a.acoustic_out + (size_t)orow * VT_DIM + 8 * (lane + 64 * i));
+    /* final RMSNorm of token 0 of each branch (rows 0 and 3), then the 36-wide projection
+     * (voxtral_tts_acoustic.c:255-261); every workgroup normalises for itself */
+    float v[2][3];
 #pragma unroll
-            for (int j = 0; j < 3; j++) {
-                v[b][j] = a.tok_in[(size_t)(3 * b) * VT_DIM + t + 1024 * j];
-                ss = fmaf(v[b][j], v[b][j], ss);
-            }
-            ss = vt_wave_sum(ss);
-            if (lane == 0) red[b][wave] = ss;
-        }
-        __syncthreads();
-        if (t < 2) {
-            float tot = 0.f;
-            for (int w = 0; w < 16; w++) tot += red[t][w];
-            s_inv[t] = 1.0f / sqrtf(tot / (float)VT_DIM + VT_EPS);
-        }
-        __syncthreads();
+    for (int b = 0; b < 2; b++) {
+        float ss = 0.f;
 #pragma unroll
         for (int j = 0; j < 3; j++) {
-            const float g = a.norm[t + 1024 * j];
-            s_xn[0][t + 1024 * j] = __fmul_rn(__fmul_rn(v[0][j], s_inv[0]), g);
-            s_xn[1][t + 1024 * j] = __fmul_rn(__fmul_rn(v[1][j], s_inv[1]), g);
+            v[b][j] = a.tok_in[(size_t)(3 * b) * VT_DIM + t + 1024 * j];
+            ss = fmaf(v[b][j], v[b][j], ss);
         }
-        __syncthreads();
-        for (int o = wave; o < 2 * VT_AC_DIM_IN; o += 16) {
-            const int b = o / VT_AC_DIM_IN, r = o % VT_AC_DIM_IN;
-            float acc = 0.f;
-#pragma unroll
-            for (int i = 0; i < VT_DIM / 512; i++) {
-                const int c = 8 * (lane + 64 * i);
-                const u32x4 w = *reinterpret_cast<const u32x4 *>(a.acoustic_out + (size_t)r * VT_DIM + c);
-                const f32x4 xa = *reinterpret_cast<const f32x4 *>(&s_xn[b][c]);
-                const f32x4 xb = *reinterpret_cast<const f32x4 *>(&s_xn[b][c + 4]);
-                acc = vt_dot8(w, xa, xb, acc);
-            }
-            acc = vt_wave_sum(acc);
-            if (lane == 0) { s_vel[o] = acc; a.vel[o] = acc; }
-        }
-        __syncthreads();
-    }
-    if (a.do_euler && t < VT_AC_DIM_IN) {
-        /* x += (1.2*vc + (1-1.2)*vu) * dt, each product rounded (voxtral_tts_acoustic.c:350-354) */
-        const float p = __fmul_rn(1.2f, s_vel[t]);
-        const float q = __fmul_rn(1.0f - 1.2f, s_vel[VT_AC_DIM_IN + t]);
-        const float xn = __fadd_rn(s_x[t], __fmul_rn(__fadd_rn(p, q), a.dt));
-        s_x[t] = xn;
-        a.x[t] = xn;
+        ss = vt_wave_sum(ss);
+        if (lane == 0) red[b][wave] = ss;
     }
     __syncthreads();
-    if (a.do_fsq && t < VT_AC_DIM_IN) {
-        /* voxtral_tts_acoustic.c:358-372 */
-        float v = s_x[t];
-        if (v > 1.0f) v = 1.0f;
-        if (v < -1.0f) v = -1.0f;
-        const float scaled = __fmul_rn(__fdiv_rn(__fadd_rn(v, 1.0f), 2.0f), 20.0f);
-        int c = (int)__fadd_rn(scaled, 0.5f);
-        if (c < 0) c = 0;
-        if (c > 20) c = 20;
-        a.codes[t + 1] = c + 2;
+    if (t < 2) {
+        float tot = 0.f;
+        for (int k = 0; k < 16; k++) tot += red[t][k];
+        s_inv[t] = 1.0f / sqrtf(tot / (float)VT_DIM + VT_EPS);
     }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const float g = a.norm[t + 1024 * j];
+        s_xn[0][t + 1024 * j] = __fmul_rn(__fmul_rn(v[0][j], s_inv[0]), g);
+        s_xn[1][t + 1024 * j] = __fmul_rn(__fmul_rn(v[1][j], s_inv[1]), g);
+    }
+    __syncthreads();
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < VT_DIM / 512; i++) {
+        const int c = 8 * (lane + 64 * i);
+        const f32x4 xa = *reinterpret_cast<const f32x4 *>(&s_xn[ob][c]);
+        const f32x4 xb = *reinterpret_cast<const f32x4 *>(&s_xn[ob][c + 4]);
+        acc = vt_dot8(w[i], xa, xb, acc);
+    }
+    acc = vt_wave_sum(acc);
+    if (mine && lane == 0) a.vel[o] = acc;
+}
+
+__global__ void __launch_bounds__(1024)
+vt_ac_edge_front_kernel(ac_edge_args a) {
+    __shared__ float s_vel[2 * VT_AC_DIM_IN];
+    __shared__ float s_x[VT_AC_DIM_IN];
+    const int t = (int)threadIdx.x;
+    const int c = t + 1024 * (int)blockIdx.x;            /* this thread's token column */
+    /* the column's row of the input projection does not depend on the latent: requested first */
+    u32x2 wr[VT_AC_DIM_IN / 4];
+    if (a.do_front) {
+        const u32x2 *p = reinterpret_cast<const u32x2 *>(a.input_proj + (size_t)c * VT_AC_DIM_IN);
+#pragma unroll
+        for (int k4 = 0; k4 < VT_AC_DIM_IN / 4; k4++) wr[k4] = p[k4];
+    }
+    if (t < VT_AC_DIM_IN) s_x[t] = a.x_in[t];
+    if (a.do_euler && t < 2 * VT_AC_DIM_IN) s_vel[t] = a.vel[t];
+    __syncthreads();
+    if (t < VT_AC_DIM_IN) {
+        float xn = s_x[t];
+        if (a.do_euler) {
+            /* x += (1.2*vc + (1-1.2)*vu) * dt, each product rounded (voxtral_tts_acoustic.c:350-354) */
+            const float p = __fmul_rn(1.2f, s_vel[t]);
+            const float q = __fmul_rn(1.0f - 1.2f, s_vel[VT_AC_DIM_IN + t]);
+            xn = __fadd_rn(xn, __fmul_rn(__fadd_rn(p, q), a.dt));
+        }
+        s_x[t] = xn;
+        if (blockIdx.x == 0) {
+            a.x_out[t] = xn;
+            if (a.do_fsq) {
+                /* voxtral_tts_acoustic.c:358-372 */
+                float v = xn;
+                if (v > 1.0f) v = 1.0f;
+                if (v < -1.0f) v = -1.0f;
+                const float scaled = __fmul_rn(__fdiv_rn(__fadd_rn(v, 1.0f), 2.0f), 20.0f);
+                int q = (int)__fadd_rn(scaled, 0.5f);
+                if (q < 0) q = 0;
+                if (q > 20) q = 20;
+                a.codes[t + 1] = q + 2;
+            }
+        }
+    }
+    __syncthreads();
     if (a.do_front) {
         /* tokens of both branches: [noise, time, llm] and [noise, time, 0]; the noise token is
          * the 36-term input projection in the CPU order (voxtral_tts_kernels.c:152-185) */
+        float acc = 0.f;
 #pragma unroll
-        for (int j = 0; j < 3; j++) {
-            const int c = t + 1024 * j;
-            const u32x2 *wr = reinterpret_cast<const u32x2 *>(a.input_proj + (size_t)c * VT_AC_DIM_IN);
-            float acc = 0.f;
-#pragma unroll
-            for (int k4 = 0; k4 < VT_AC_DIM_IN / 4; k4++) {
-                const u32x2 w = wr[k4];
-                acc = __fadd_rn(acc, __fmul_rn(vt_bf16_lo(w.x), s_x[4 * k4]));
-                acc = __fadd_rn(acc, __fmul_rn(vt_bf16_hi(w.x), s_x[4 * k4 + 1]));
-                acc = __fadd_rn(acc, __fmul_rn(vt_bf16_lo(w.y), s_x[4 * k4 + 2]));
-                acc = __fadd_rn(acc, __fmul_rn(vt_bf16_hi(w.y), s_x[4 * k4 + 3]));
-            }
-            const float tm = a.time_tok[c];
-            a.tok_out[c] = acc;
-            a.tok_out[VT_DIM + c] = tm;
-            a.tok_out[2 * VT_DIM + c] = a.llm_tok[c];
-            a.tok_out[3 * VT_DIM + c] = acc;
-            a.tok_out[4 * VT_DIM + c] = tm;
-            a.tok_out[5 * VT_DIM + c] = 0.f;
+        for (int k4 = 0; k4 < VT_AC_DIM_IN / 4; k4++) {
+            const u32x2 w = wr[k4];
+            acc = __fadd_rn(acc, __fmul_rn(vt_bf16_lo(w.x), s_x[4 * k4]));
+            acc = __fadd_rn(acc, __fmul_rn(vt_bf16_hi(w.x), s_x[4 * k4 + 1]));
+            acc = __fadd_rn(acc, __fmul_rn(vt_bf16_lo(w.y), s_x[4 * k4 + 2]));
+            acc = __fadd_rn(acc, __fmul_rn(vt_bf16_hi(w.y), s_x[4 * k4 + 3]));
         }
+        const float tm = a.time_tok[c];
+        a.tok_out[c] = acc;
+        a.tok_out[VT_DIM + c] = tm;
+        a.tok_out[2 * VT_DIM + c] = a.llm_tok[c];
+        a.tok_out[3 * VT_DIM + c] = acc;
+        a.tok_out[4 * VT_DIM + c] = tm;
+        a.tok_out[5 * VT_DIM + c] = 0.f;
     }
 }
 
@@ -499,7 +528,7 @@ __global__ void __launch_bounds__(1024) vt_semantic_argmax_kernel(const float *l
 
 /* device work area of the acoustic path, in floats */
 struct ac_work {
-    float *tok, *qkv, *h, *llm_tok, *hidden, *x, *vel, *temb, *time_tok1, *logits;
+    float *tok, *qkv, *h, *llm_tok, *hidden, *x, *x2, *vel, *temb, *time_tok1, *logits;
     int *codes;
 };
 #define AC_WORK_FLOATS (AC_ROWS * (VT_DIM + VT_QKV_DIM + VT_FFN) + 4 * VT_DIM + 64 + 128 + VT_SEM_PADDED + 64)
@@ -514,6 +543,7 @@ static void carve(ac_work *w, float *base) {
     w->time_tok1 = w->temb + VT_DIM;
     w->x = w->time_tok1 + VT_DIM;
     w->vel = w->x + 64;
+    w->x2 = w->vel + 80;                                 /* vel uses 72 of its 128 floats */
     w->logits = w->vel + 128;
     w->codes = (int *)(w->logits + VT_SEM_PADDED);
 }
@@ -573,14 +603,22 @@ float vt_bench_acoustic_phase(int phase, int iters) {
     return ms / (float)iters;
 }
 
+/* One step boundary.  The latent ping-pongs between w->x and w->x2: `flip` counts the front
+ * launches of the frame so far; the caller keeps it. */
 static void launch_edge(const ac_work *w, const float *time_tok, const float *llm_tok, float dt, int back, int euler,
-                        int front, int fsq) {
+                        int front, int fsq, int *flip) {
     const vt_acoustic_dev *ac = &g_vt.ac;
     ac_edge_args a;
     a.tok_in = w->tok; a.tok_out = w->tok; a.norm = ac->norm; a.acoustic_out = ac->acoustic_out;
-    a.input_proj = ac->input_proj; a.time_tok = time_tok; a.llm_tok = llm_tok; a.x = w->x; a.vel = w->vel;
-    a.codes = w->codes; a.dt = dt; a.do_back = back; a.do_euler = euler; a.do_front = front; a.do_fsq = fsq;
-    hipLaunchKernelGGL(vt_ac_edge_kernel, dim3(1), dim3(1024), 0, g_vt.stream, a);
+    a.input_proj = ac->input_proj; a.time_tok = time_tok; a.llm_tok = llm_tok; a.vel = w->vel;
+    a.codes = w->codes; a.dt = dt; a.do_euler = euler; a.do_front = front; a.do_fsq = fsq;
+    a.x_in = (*flip & 1) ? w->x2 : w->x;
+    a.x_out = (*flip & 1) ? w->x : w->x2;
+    if (back) hipLaunchKernelGGL(vt_ac_edge_back_kernel, dim3(AC_BACK_WGS), dim3(1024), 0, g_vt.stream, a);
+    if (euler || front || fsq) {
+        hipLaunchKernelGGL(vt_ac_edge_front_kernel, dim3(front ? AC_FRONT_WGS : 1), dim3(1024), 0, g_vt.stream, a);
+        *flip += 1;
+    }
 }
 
 /* Host evaluation of the sinusoidal time embedding with libm, in the order of
@@ -670,9 +708,10 @@ static void predict(float *out_c, float *out_u, const float *x_t, const float *l
         s_memo.hidden_valid = 1;
     }
     VT_TRYV(hipMemcpyAsync(w.x, x_t, sizeof(float) * VT_AC_DIM_IN, hipMemcpyDefault, st));
-    launch_edge(&w, time_tok, llm_tok, 0.f, 0, 0, 1, 0);
+    int flip = 0;
+    launch_edge(&w, time_tok, llm_tok, 0.f, 0, 0, 1, 0, &flip);
     if (run_layers(&w)) return;
-    launch_edge(&w, time_tok, llm_tok, 0.f, 1, 0, 0, 0);
+    launch_edge(&w, time_tok, llm_tok, 0.f, 1, 0, 0, 0, &flip);
     VT_TRYV(hipGetLastError());
     VT_TRYV(hipStreamSynchronize(st));
     float vel[2 * VT_AC_DIM_IN];
@@ -715,12 +754,13 @@ static int enqueue_frame(ac_work *w, const float *d_or_h_hidden, const float *x0
     hipLaunchKernelGGL(vt_semantic_argmax_kernel, dim3(1), dim3(1024), 0, st, w->logits, w->codes);
     vt_launch_linear(w->llm_tok, w->hidden, ac->llm_proj, NULL, 1, VT_DIM, VT_DIM);
     /* the flow runs without waiting for the semantic code; an END_AUDIO frame discards it */
-    launch_edge(w, ac->time_tok, w->llm_tok, 0.f, 0, 0, 1, 0);
+    int flip = 0;                                        /* 1 + AC_STEPS front launches: the latent ends in w->x */
+    launch_edge(w, ac->time_tok, w->llm_tok, 0.f, 0, 0, 1, 0, &flip);
     for (int s = 0; s < AC_STEPS; s++) {
         volatile float dt = ts[s + 1] - ts[s];
         if (run_layers(w)) return -1;
         const int last = s + 1 == AC_STEPS;
-        launch_edge(w, ac->time_tok + (size_t)(last ? s : s + 1) * VT_DIM, w->llm_tok, (float)dt, 1, 1, !last, last);
+        launch_edge(w, ac->time_tok + (size_t)(last ? s : s + 1) * VT_DIM, w->llm_tok, (float)dt, 1, 1, !last, last, &flip);
     }
     return vt_check(hipGetLastError(), "frame launch");
 }
