@@ -576,12 +576,108 @@ def bench_matvec(args):
     print(json.dumps(out))
 
 
+def bench_layer(args):
+    """configs[1]: one decoder layer, decode step at batch 1 over a KV cache of 512 positions
+    ~N(0,1).  A step is one tts_hip_layer_decode on a device-resident hidden state (the whole-step
+    kernel run over a single layer, final norm off)."""
+    import cases
+    K, W = args.steps, args.warmup
+    pos, kv_max = 512, 520
+    layer = S.Layer(3)
+    ones = np.ones(S.DIM, np.float32)
+    k = np.zeros((N_LAYERS, kv_max, S.KV_DIM), np.float32)
+    v = np.zeros((N_LAYERS, kv_max, S.KV_DIM), np.float32)
+    k[0, :pos] = S.f32_normal((pos, S.KV_DIM), 200)
+    v[0, :pos] = S.f32_normal((pos, S.KV_DIM), 300)
+    x = S.f32_normal(S.DIM, 42)
+    hip = H.Hip(kv_max=kv_max)
+    lib = hip.lib
+    hip.upload_decoder([layer], ones, 1)
+    hip.set_kv(k, v)
+    lib.tts_hip_set_decode_mode(args.mode)
+    d_x = H.DevBuf.from_numpy(lib, x)
+    lib.tts_hip_layer_decode(0, d_x.ptr, pos)
+    lib.tts_hip_sync()
+    hip.check()
+    got = d_x.to_numpy(np.float32, (S.DIM,))
+    d_in = H.DevBuf.from_numpy(lib, x)
+    for _ in range(W):
+        lib.tts_hip_to_device(d_x.ptr, x.ctypes.data, x.nbytes)
+        lib.tts_hip_layer_decode(0, d_x.ptr, pos)
+    lib.tts_hip_sync()
+    # the hidden state is fed back in place: values drift but the bytes moved do not depend on them
+    lib.tts_hip_to_device(d_x.ptr, x.ctypes.data, x.nbytes)
+    lib.tts_hip_timer_start()
+    for _ in range(K):
+        lib.tts_hip_layer_decode(0, d_x.ptr, pos)
+    ms = lib.tts_hip_timer_stop_ms() / K
+    hip.check()
+    nbytes = LAYER_WEIGHT_BYTES + 2 * S.DIM * 4 + 2 * (pos + 1) * S.KV_DIM * 4 + 2 * S.KV_DIM * 4 + 2 * S.DIM * 4
+    gbps = nbytes / ms / 1e6
+    out = {
+        "metric": "one decoder layer, decode step ms (512 cached positions)",
+        "value": round(ms * 1e3, 2), "unit": "us/step",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(ms, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "one Mistral decoder layer, decode step at batch 1, KV cache of 512 positions ~N(0,1), "
+                               "hidden ~N(0,1) (BASELINE.json configs[1])",
+                   "weights": "bf16 N(0,0.02) seeded, truncated", "activations": "f32",
+                   "schedule": {0: "persistent whole-step kernel over one layer", 1: "one kernel per phase",
+                                2: "streaming kernel"}.get(args.mode, str(args.mode)),
+                   "timed": "events on the library's stream, back-to-back launches, operands resident in HBM"},
+        "hbm_gbps": round(gbps, 1),
+        "roofline": {"kernel": "vt_decode_step_kernel (one layer)", "bound": "hbm", "achieved": round(gbps, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_per_launch": nbytes, "ms_per_launch": round(ms, 5)},
+        "cpu_baseline": None,
+    }
+    if args.cpu_seconds > 0:
+        kind = "reference" if S.have_ref() else "port"
+        if S.have_ref():
+            b = cases.RefBackend()
+            b.llm_open([layer] * N_LAYERS, ones, kv_max)
+            nb = N_LAYERS * kv_max * S.KV_DIM * 4
+            C.memmove(b.lib.ref_kv_k(b.ctx), k.ctypes.data, nb)
+            C.memmove(b.lib.ref_kv_v(b.ctx), v.ctypes.data, nb)
+            b.lib.ref_set_kv_len(b.ctx, pos)
+            t0 = time.time()
+            b.llm_forward(x)                                   # 26 layers: the reference has no per-layer entry
+            cpu_ms = (time.time() - t0) * 1e3 / N_LAYERS
+            b.llm_close()
+            sample = "one tts_llm_forward over 26 copies of the layer at pos 512, divided by 26"
+        else:
+            b = cases.OracleBackend(threads=1)
+            b.llm_open([layer], ones, kv_max, n_layers=1)
+            b.kv_k[0], b.kv_v[0] = k[0], v[0]
+            b.pos = pos
+            t0 = time.time()
+            b.llm_forward(x)
+            cpu_ms = (time.time() - t0) * 1e3
+            sample = "one layer step of the CPU port at pos 512"
+        out["cpu_baseline"] = {"value": round(cpu_ms * 1e3, 0), "unit": "us/step", "cores": 1, "kind": kind,
+                               "sample": sample, "gbps": round(nbytes / cpu_ms / 1e6, 2)}
+        # parity of the timed entry point against the CPU port: the port's hidden state is the final
+        # norm (unit gains) of the residual stream that tts_hip_layer_decode leaves
+        o = cases.OracleBackend(threads=8)
+        o.llm_open([layer], ones, kv_max, n_layers=1)
+        o.kv_k[0], o.kv_v[0] = k[0], v[0]
+        o.pos = pos
+        ref_h = o.llm_forward(x)
+        renorm = o.rms_norm(got.reshape(1, -1), ones, 1)[0]
+        mx, l2 = S.rel_errors(ref_h, renorm)
+        out["parity"] = {"max_abs_over_rms": float(f"{mx:.3g}"), "rel_l2": float(f"{l2:.3g}"), "against": "port"}
+        assert mx < 1e-3 and l2 < 1e-3, (mx, l2)
+    hip.close()
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=("decode", "prefill", "acoustic", "frame", "codec", "matvec"), default="decode",
+    ap.add_argument("--workload", choices=("decode", "prefill", "acoustic", "frame", "codec", "matvec", "layer"), default="decode",
                     help="decode = the headline metric; prefill / acoustic = the other two configurations")
     ap.add_argument("--mode", type=int, default=0, help="0 persistent kernel, 1 per-phase kernels, 2 streaming kernel")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
@@ -605,6 +701,8 @@ def main():
         return bench_frame(args)
     if args.workload == "matvec":
         return bench_matvec(args)
+    if args.workload == "layer":
+        return bench_layer(args)
     K, W = args.steps, args.warmup
     workers = min(16, os.cpu_count() or 8)
 
