@@ -787,6 +787,19 @@ def main():
     lib.tts_hip_sync()
     hip.check()
 
+    # the drop-in entry point with host pointers (12 KB up, 12 KB down and one synchronisation per
+    # step, as voxtral_tts_llm.c calls it): wall clock over the same positions, reported beside `value`
+    pos = pos0
+    e_host = d_e.to_numpy(np.float32, S.DIM)
+    h_host = np.zeros(S.DIM, np.float32)
+    n_host = min(K, 50)
+    lib.tts_hip_llm_forward(h_host.ctypes.data, e_host.ctypes.data, pos)
+    t0 = time.perf_counter()
+    for i in range(n_host):
+        lib.tts_hip_llm_forward(h_host.ctypes.data, e_host.ctypes.data, pos + i)
+    ms_host = (time.perf_counter() - t0) * 1e3 / n_host
+    hip.check()
+
     avg_pos = pos0 + (K - 1) / 2.0
     bytes_launch = step_bytes(avg_pos)
     achieved = bytes_launch / (ms_kernel * 1e-3) / 1e9
@@ -813,6 +826,7 @@ def main():
         "hbm_gbps": round((bytes_launch + 2 * S.DIM * S.DIM) / (ms_step * 1e-3) / 1e9, 1),
         "hbm_frac_of_peak": round((bytes_launch + 2 * S.DIM * S.DIM) / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
         "ms_per_frame_normalised_6p8GB": round(ms_kernel * 6.8e9 / bytes_launch, 4),
+        "ms_per_frame_host_pointers": round(ms_host, 4),
         "roofline": {
             "kernel": ("vt_decode_step_kernel", "5 phase kernels per layer", "vt_decode_stream_kernel")[args.mode],
             "bound": "hbm",
