@@ -113,6 +113,21 @@ def test_config1_matvec_shapes(hip, orc, n, k):
     assert ok, (mr, ma, bad)
 
 
+@pytest.mark.parametrize("n,k", [(1000, 512), (5, 1024), (777, 2560), (257, 9216), (300, 16384), (64, 520)])
+def test_matvec_ragged_shapes(hip, orc, n, k):
+    """Single-row products whose rows do not divide over the workgroups, with one or many 512-wide
+    chunks per row; 16384 columns do not fit the stream kernel's LDS and 520 are not whole chunks:
+    those two take the wave-per-row kernel."""
+    W = S.bf16_normal((n, k), 31 * n + k)
+    x = S.f32_normal((1, k), 17)
+    ref = orc.linear(x, W, None, 1)
+    got = _linear(hip, x, W, 1, True)
+    mx, l2 = S.rel_errors(ref, got)
+    assert mx < 1e-3 and l2 < 1e-3, (n, k, mx, l2)
+    again = _linear(hip, x, W, 1, True)
+    assert np.array_equal(got, again)              # fixed summation order: reproducible
+
+
 @pytest.mark.parametrize("seq", [3, 6, 19])
 def test_linear_several_rows_and_host_weights(hip, orc, seq):
     W = S.bf16_normal((200, 3072), 77)
