@@ -99,6 +99,34 @@ def test_malformed_files_are_errors(lib, tmp_path):
     assert probe(lib, p, "x")[0] == 1
 
 
+def test_hostile_headers_stay_inside_the_file(lib, tmp_path):
+    """Numbers are read with every character checked against the end of the header (it is not
+    NUL-terminated and may end where the file ends), nesting is bounded, and shapes whose
+    product does not fit are not multiplied out."""
+    n0 = lib.tts_hip_error_count()
+    # the header, and with it the file, ends in the middle of a number
+    p = tmp_path / "digits.safetensors"
+    raw_file(p, b'{"x":{"dtype":"F32","shape":[4],"data_offsets":[0,1' + b"6" * 4000)
+    assert probe(lib, p, "x")[0] == -1
+    # a number that does not fit 63 bits
+    p = tmp_path / "big.safetensors"
+    raw_file(p, b'{"x":{"dtype":"F32","shape":[4],"data_offsets":[0,99999999999999999999999]}}', b"\0" * 16)
+    assert probe(lib, p, "x")[0] == -1
+    # metadata nested deeper than any writer produces
+    p = tmp_path / "deep.safetensors"
+    raw_file(p, b'{"__metadata__":' + b"[" * 100000 + b"]" * 100000 + b"}")
+    assert probe(lib, p, "x")[0] == -1
+    assert lib.tts_hip_error_count() == n0 + 3
+    # negative offsets and extents: malformed / a tensor that matches no expected size
+    p = tmp_path / "neg.safetensors"
+    raw_file(p, {"x": {"dtype": "F32", "shape": [4], "data_offsets": [-16, 0]}}, b"\0" * 16)
+    assert probe(lib, p, "x")[0] == -1
+    p = tmp_path / "huge.safetensors"
+    raw_file(p, {"x": {"dtype": "BF16", "shape": [1 << 40, 1 << 40, -3], "data_offsets": [0, 16]}}, b"\0" * 16)
+    rc, dtype, rank, shape, nbytes = probe(lib, p, "x")
+    assert (rc, dtype, rank, nbytes) == (0, "BF16", 3, 16)          # the header itself is well-formed
+
+
 def test_load_needs_an_initialised_backend(lib, tmp_path):
     n0 = lib.tts_hip_error_count()
     p = tmp_path / "e.safetensors"

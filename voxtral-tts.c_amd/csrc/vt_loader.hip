@@ -63,20 +63,26 @@ static int st_string(st_cur *c, char *out, size_t cap) {
     return 0;
 }
 
+/* decimal integer; the header is not NUL-terminated, so every character is checked against its end */
 static int st_int(st_cur *c, long long *v) {
     st_ws(c);
-    char *e;
-    const long long x = strtoll(c->p, &e, 10);
-    if (e == c->p) return -1;
-    c->p = e;
-    *v = x;
+    int neg = 0;
+    if (c->p < c->end && *c->p == '-') { neg = 1; c->p++; }
+    if (c->p >= c->end || *c->p < '0' || *c->p > '9') return -1;
+    long long x = 0;
+    while (c->p < c->end && *c->p >= '0' && *c->p <= '9') {
+        if (x > (0x7fffffffffffffffLL - 9) / 10) return -1;          /* would not fit */
+        x = x * 10 + (*c->p++ - '0');
+    }
+    *v = neg ? -x : x;
     return 0;
 }
 
-/* skips any JSON value */
-static int st_skip(st_cur *c) {
+/* skips any JSON value; nesting beyond ST_MAX_DEPTH is refused (the recursion is on the C stack) */
+#define ST_MAX_DEPTH 32
+static int st_skip_at(st_cur *c, int depth) {
     st_ws(c);
-    if (c->p >= c->end) return -1;
+    if (c->p >= c->end || depth > ST_MAX_DEPTH) return -1;
     if (*c->p == '"') return st_string(c, NULL, 0);
     if (*c->p == '{' || *c->p == '[') {
         const char open = *c->p, close = open == '{' ? '}' : ']';
@@ -84,7 +90,7 @@ static int st_skip(st_cur *c) {
         if (st_eat(c, close)) return 0;
         for (;;) {
             if (open == '{') { if (st_string(c, NULL, 0) || !st_eat(c, ':')) return -1; }
-            if (st_skip(c)) return -1;
+            if (st_skip_at(c, depth + 1)) return -1;
             if (st_eat(c, ',')) continue;
             return st_eat(c, close) ? 0 : -1;
         }
@@ -92,6 +98,7 @@ static int st_skip(st_cur *c) {
     while (c->p < c->end && *c->p != ',' && *c->p != '}' && *c->p != ']') c->p++;
     return 0;
 }
+static int st_skip(st_cur *c) { return st_skip_at(c, 0); }
 
 static int st_entry(st_cur *c, st_tensor *t) {
     if (!st_eat(c, '{')) return -1;
@@ -191,10 +198,17 @@ static const st_tensor *st_find(const st_file *f, const char *name) {
     return NULL;
 }
 
+/* number of elements, or -1 for shapes that no tensor of this model has (rank above 4, a
+ * negative extent, a product beyond 2^40) */
 static long long st_count(const st_tensor *t) {
+    if (t->rank > 4) return -1;
     long long n = 1;
-    for (int i = 0; i < t->rank && i < 4; i++) n *= t->shape[i];
-    return t->rank > 4 ? -1 : n;
+    for (int i = 0; i < t->rank; i++) {
+        const long long d = t->shape[i];
+        if (d < 0 || (d > 0 && n > (1LL << 40) / d)) return -1;
+        n *= d;
+    }
+    return n;
 }
 
 /* bf16 tensor of exactly `elems` elements, straight out of the mapping */
