@@ -349,7 +349,9 @@ __device__ __forceinline__ void vt_attn_geometry(int n, int nch_max, int nw, int
  * positions) has all its K and V rows requested before any is used.  Each of the 32 lane
  * groups keeps its own online-softmax state; they are merged through LDS at the end.  The
  * four workgroups of a kv head sit on one XCD (blockIdx % 8) and share its rows in that L2. */
-#define VT_ATT_DIRECT_MAX 512
+#ifndef VT_ATT_DIRECT_MAX
+#define VT_ATT_DIRECT_MAX 960      /* measured crossover with the chunked schedule: between 900 and 1024 positions */
+#endif
 
 /* K and V rows of one batch: 4 rounds of one position per lane group */
 struct vt_att_rows { f32x4 ka[4], kb[4], va[4], vb[4]; };
