@@ -18,6 +18,10 @@
 
 #ifdef USE_CUDA
 
+/* the context type of the exported global; only kv_cache_k_gpu / kv_cache_v_gpu / kv_cache_max /
+ * initialized are read from outside the backend (voxtral_tts_llm.c:380-381); the per-layer
+ * device pointers of tts_cuda_layer_weights_t are private to the backend and have no alias */
+#define tts_cuda_ctx_t                      tts_hip_ctx_t
 #define g_cuda                              g_hip
 #define tts_cuda_init                       tts_hip_init
 #define tts_cuda_upload_llm_weights         tts_hip_upload_llm_weights
