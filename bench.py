@@ -690,7 +690,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus above 1 is not supported "
-                 "(the decode chain is not sharded; see DESIGN.md)")
+                 "(batch-1 decode is one dependent chain of layers and is not sharded)")
     if args.workload == "prefill":
         return bench_prefill(args)
     if args.workload == "acoustic":
