@@ -63,6 +63,9 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
 
     const float *x_in = a.in_embed;
     vt_qkv_prefetch(ring, a.layers[0]);
+    /* scalars of the whole step: who runs the attention, and whether enough workgroups are left over */
+    const int att_busy = __builtin_amdgcn_readfirstlane(vt_attn_busy(a));
+    const bool l2_prefetch = 4 * att_busy <= 3 * (int)gridDim.x;
     for (int l = 0; l < a.n_layers; l++) {
         const vt_layer_dev L = a.layers[l];
         /* the next phase's first row is requested as soon as the ring is free, the other rows
@@ -77,9 +80,12 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
         const int wo_slots = vt_wo_rows().nr * 4 <= VT_WO_SLOTS ? VT_WO_SLOTS : VT_RING;
         if (!vt_barrier_then(gs, &s_flag, [&] {
                 vt_w13_prefetch(ring, L, VT_PART_ALL, wo_slots, VT_RING);
-                if (vt_attn_is_direct(a)) {
-                    vt_w13_l2_prefetch(L);
-                    if (more) vt_kv_l2_prefetch(a, l + 1);
+                /* the workgroups without a share of the attention prefetch into their L2: gate|up rows
+                 * when at least a quarter of the grid is free, the next layer's K/V rows while the
+                 * cache is short enough to leave room for them */
+                if (l2_prefetch) {
+                    vt_w13_l2_prefetch(L, att_busy);
+                    if (more && vt_attn_is_direct(a)) vt_kv_l2_prefetch(a, l + 1, att_busy);
                 }
             }, tn))
             return;

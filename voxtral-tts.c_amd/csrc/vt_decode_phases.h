@@ -29,7 +29,9 @@
 
 #define VT_RING 18            /* 16-byte buffers per lane in the row ring */
 #define VT_ATT_STRIDE 132     /* floats per attention partial: m, l, pad, pad, o[128] */
-#define VT_ATT_MIN_CHUNK 32   /* positions per attention workgroup before the cache is split further */
+#ifndef VT_ATT_MIN_CHUNK
+#define VT_ATT_MIN_CHUNK 64   /* positions per attention workgroup before the cache is split further */
+#endif
 #define VT_LDS_X 9216         /* staged activation vector (largest: the SwiGLU output) */
 #define VT_LDS_Y 512          /* row results of one workgroup */
 #define VT_LDS_FLOATS (VT_LDS_X + VT_LDS_Y)
@@ -350,7 +352,7 @@ __device__ __forceinline__ void vt_attn_geometry(int n, int nch_max, int nw, int
  * groups keeps its own online-softmax state; they are merged through LDS at the end.  The
  * four workgroups of a kv head sit on one XCD (blockIdx % 8) and share its rows in that L2. */
 #ifndef VT_ATT_DIRECT_MAX
-#define VT_ATT_DIRECT_MAX 960      /* measured crossover with the chunked schedule: between 900 and 1024 positions */
+#define VT_ATT_DIRECT_MAX 768      /* measured crossover with the chunked schedule (1.390 against 1.393 ms/frame at 768) */
 #endif
 
 /* K and V rows of one batch: 4 rounds of one position per lane group */
@@ -445,10 +447,10 @@ __device__ __forceinline__ void vt_attn_direct(const vt_step_args &a, int layer,
  * and kv head) and nothing else allocates in L2 in between - weights stream with the
  * non-temporal hint - so the next attention finds them there instead of in HBM.  Wave 0 stays
  * out of it: it polls the barrier. */
-__device__ __forceinline__ void vt_kv_l2_prefetch(const vt_step_args &a, int layer) {
+__device__ __forceinline__ void vt_kv_l2_prefetch(const vt_step_args &a, int layer, int busy) {
     const int G = (int)gridDim.x, wg = (int)blockIdx.x, nw = (int)(blockDim.x >> 6);
-    if ((G & 7) || wg < VT_HEADS || vt_wave() == 0) return;
-    const int idle0 = VT_HEADS >> 3;                            /* workgroups per XCD that run the attention */
+    if ((G & 7) || wg < busy || vt_wave() == 0) return;
+    const int idle0 = busy >> 3;                                /* workgroups per XCD that run the attention */
     const int me = (((wg >> 3) - idle0) * (nw - 1) + vt_wave() - 1) * VT_WAVE + vt_lane();
     const int n_lanes = ((G >> 3) - idle0) * (nw - 1) * VT_WAVE;
     const int lines_per_row = VT_HEAD_DIM * 4 / 128;            /* 4 */
@@ -461,6 +463,16 @@ __device__ __forceinline__ void vt_kv_l2_prefetch(const vt_step_args &a, int lay
         acc ^= *reinterpret_cast<const unsigned *>(p);
     }
     asm volatile("" ::"v"(acc));
+}
+
+/* Workgroups 0 .. busy-1 run the attention of this step (busy is a multiple of 8: the same number
+ * on every XCD); the others have the phase to themselves and prefetch into their L2. */
+__device__ __forceinline__ int vt_attn_busy(const vt_step_args &a) {
+    if (vt_attn_is_direct(a)) return VT_HEADS;
+    const int nch_max = (int)gridDim.x / VT_KV_HEADS;
+    int cs, nch;
+    vt_attn_geometry(a.pos + 1, nch_max, (int)(blockDim.x >> 6), cs, nch);
+    return nch * VT_KV_HEADS;
 }
 
 __device__ __forceinline__ void vt_attn_phase(const vt_step_args &a, int layer, float *lds) {
@@ -635,10 +647,10 @@ __device__ __forceinline__ void vt_w13_prefetch(u32x4 (&ring)[VT_RING], const vt
 #define VT_L2_SKIP 24          /* lines of the first prefetched row that are left out: 1.5 rows fit the L2 as well as 2 */
 #endif
 
-__device__ __forceinline__ void vt_w13_l2_prefetch(const vt_layer_dev &L) {
+__device__ __forceinline__ void vt_w13_l2_prefetch(const vt_layer_dev &L, int busy) {
     const int G = (int)gridDim.x, wg = (int)blockIdx.x, nw = (int)(blockDim.x >> 6);
-    if ((G & 7) || wg < VT_HEADS || vt_wave() == 0) return;
-    const int per_x = G >> 3, idle0 = VT_HEADS >> 3;
+    if ((G & 7) || wg < busy || vt_wave() == 0) return;
+    const int per_x = G >> 3, idle0 = busy >> 3;
     const int me = (((wg >> 3) - idle0) * (nw - 1) + vt_wave() - 1) * VT_WAVE + vt_lane();
     const int n_lanes = (per_x - idle0) * (nw - 1) * VT_WAVE;
     int per_wg = (2 * VT_FFN + G - 1) / G;
