@@ -337,7 +337,8 @@ __device__ __forceinline__ void vt_qkv_body(u32x4 (&ring)[VT_RING], const vt_lay
  * voxtral_tts_kernels.c:426-462). */
 __device__ __forceinline__ void vt_attn_geometry(int n, int nch_max, int nw, int &cs, int &nch) {
     nch = (n + VT_ATT_MIN_CHUNK - 1) / VT_ATT_MIN_CHUNK;
-    if (nch > nch_max) nch = nch_max;
+    /* at most three quarters of the grid: the rest prefetches gate|up rows into L2 meanwhile */
+    if (nch > nch_max * 3 / 4) nch = nch_max * 3 / 4;
     if (nch < 1) nch = 1;
     cs = (n + nch - 1) / nch;
     cs = (cs + nw - 1) / nw * nw;
