@@ -64,22 +64,28 @@ template <int PH> struct ac_shape {
 /* Activation rows are fetched into registers BEFORE the weight loads of a pass are
  * issued: a wave's loads return in order, so this way the planes can be built while
  * the weights are still streaming in. */
-struct ac_rows_regs { f32x2 v[AC_ROWS][3]; f32x2 g[3]; };
+struct ac_rows_regs { f32x4 v[AC_ROWS][2]; f32x4 g[2]; };
 struct ac_attn_regs { f32x4 q[3][4], k[3][4], v[3][4]; };
 
-/* rows of 3072: thread t owns the column pairs 2t + 1024 j */
+/* rows of 3072 = 768 groups of 4 columns: thread t owns group t, and group 512 + t when t < 256
+ * (16-byte loads: half the load instructions of 8-byte ones for the same bytes) */
 __device__ __forceinline__ void ac_fetch_rows(ac_rows_regs &r, const float *src, int src_stride,
                                               const float *gain) {
     const int t = (int)threadIdx.x;
+    const bool two = t < 256;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f}, one = {1.f, 1.f, 1.f, 1.f};
 #pragma unroll
-    for (int m = 0; m < AC_ROWS; m++)
-#pragma unroll
-        for (int j = 0; j < 3; j++)
-            r.v[m][j] = *reinterpret_cast<const f32x2 *>(src + (size_t)m * src_stride + 2 * t + 1024 * j);
-#pragma unroll
-    for (int j = 0; j < 3; j++) {
-        r.g[j] = f32x2{1.f, 1.f};
-        if (gain) r.g[j] = *reinterpret_cast<const f32x2 *>(gain + 2 * t + 1024 * j);
+    for (int m = 0; m < AC_ROWS; m++) {
+        const f32x4 *row = reinterpret_cast<const f32x4 *>(src + (size_t)m * src_stride);
+        r.v[m][0] = row[t];
+        r.v[m][1] = two ? row[512 + t] : zero;
+    }
+    r.g[0] = one;
+    r.g[1] = one;
+    if (gain) {
+        const f32x4 *g = reinterpret_cast<const f32x4 *>(gain);
+        r.g[0] = g[t];
+        r.g[1] = two ? g[512 + t] : one;
     }
 }
 
@@ -88,13 +94,17 @@ template <bool NORM>
 __device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned char *lo, int pitch,
                                                   const ac_rows_regs &r, float *red) {
     const int t = (int)threadIdx.x;
+    const bool two = t < 256;
     float inv[AC_ROWS];
     if (NORM) {
 #pragma unroll
         for (int m = 0; m < AC_ROWS; m++) {
             float ss = 0.f;
 #pragma unroll
-            for (int j = 0; j < 3; j++) ss = fmaf(r.v[m][j].x, r.v[m][j].x, fmaf(r.v[m][j].y, r.v[m][j].y, ss));
+            for (int j = 0; j < 2; j++) {
+                const f32x4 v = r.v[m][j];                     /* zeros where this thread has no second group */
+                ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+            }
             ss = vt_wave_sum(ss);
             if (vt_lane() == 0) red[vt_wave() * 8 + m] = ss;
         }
@@ -108,21 +118,27 @@ __device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned ch
         }
     }
 #pragma unroll
-    for (int j = 0; j < 3; j++) {
-        const int c = 2 * t + 1024 * j;
-        const f32x2 g = r.g[j];
+    for (int j = 0; j < 2; j++) {
+        if (j == 0 || two) {
+            const int c = 4 * (t + 512 * j);
+            const f32x4 g = r.g[j];
 #pragma unroll
-        for (int m = 0; m < AC_ROWS; m++) {
-            float a = r.v[m][j].x, b = r.v[m][j].y;
-            if (NORM) {
-                a = __fmul_rn(__fmul_rn(a, inv[m]), g.x);
-                b = __fmul_rn(__fmul_rn(b, inv[m]), g.y);
+            for (int m = 0; m < AC_ROWS; m++) {
+                f32x4 v = r.v[m][j];
+                if (NORM) {
+                    v.x = __fmul_rn(__fmul_rn(v.x, inv[m]), g.x);
+                    v.y = __fmul_rn(__fmul_rn(v.y, inv[m]), g.y);
+                    v.z = __fmul_rn(__fmul_rn(v.z, inv[m]), g.z);
+                    v.w = __fmul_rn(__fmul_rn(v.w, inv[m]), g.w);
+                }
+                unsigned h0, l0, h1, l1, h2, l2, h3, l3;
+                vt_split_planes(v.x, h0, l0);
+                vt_split_planes(v.y, h1, l1);
+                vt_split_planes(v.z, h2, l2);
+                vt_split_planes(v.w, h3, l3);
+                *reinterpret_cast<u32x2 *>(hi + m * pitch + 2 * c) = u32x2{h0 | (h1 << 16), h2 | (h3 << 16)};
+                *reinterpret_cast<u32x2 *>(lo + m * pitch + 2 * c) = u32x2{l0 | (l1 << 16), l2 | (l3 << 16)};
             }
-            unsigned h0, l0, h1, l1;
-            vt_split_planes(a, h0, l0);
-            vt_split_planes(b, h1, l1);
-            *reinterpret_cast<unsigned *>(hi + m * pitch + 2 * c) = h0 | (h1 << 16);
-            *reinterpret_cast<unsigned *>(lo + m * pitch + 2 * c) = l0 | (l1 << 16);
         }
     }
 }
