@@ -21,7 +21,7 @@ void vt_launch_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_x, size_t n)
 /* rows of 3072: x += sum of planes (splits > 0), then planes of rmsnorm(x)*w (d_w != NULL) */
 void vt_launch_residual_norm_split(float *d_x, const float *d_part, int splits, size_t part_stride,
                                    const float *d_w, uint16_t *d_hi, uint16_t *d_lo, int rows);
-/* n_out even: planes of silu(gate)*up from interleaved (gate, up) pairs */
+/* n_out a multiple of 4, tail_col0 of 8: planes of silu(gate)*up from interleaved (gate, up) pairs */
 void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, size_t n_out, int tail_col0,
                             const float *d_tail, int tail_planes, size_t tail_stride);
 void vt_launch_sum_planes(float *d_out, const float *d_part, int splits, size_t stride, size_t n);

@@ -206,22 +206,31 @@ void vt_launch_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_x, size_t n)
 __global__ void __launch_bounds__(256)
 vt_residual_norm_split_kernel(float *x, const float *part, int splits, size_t part_stride,
                               const float *w, uint16_t *hi, uint16_t *lo, float eps) {
+    /* a thread owns 4 consecutive columns at 4 (t + 256 j): 16-byte loads and stores, 8-byte plane
+     * stores (a quarter of the memory instructions of element-wise accesses) */
     __shared__ float red[4];
     const size_t row = blockIdx.x;
-    float v[VT_DIM / 256];
+    constexpr int NJ = VT_DIM / 1024;
+    f32x4 v[NJ];
     float ss = 0.f;
 #pragma unroll
-    for (int j = 0; j < VT_DIM / 256; j++) {
-        const size_t i = row * VT_DIM + threadIdx.x + 256 * j;
-        float a = x[i];
+    for (int j = 0; j < NJ; j++) {
+        const size_t i = row * VT_DIM + 4 * ((size_t)threadIdx.x + 256 * j);
+        f32x4 a = *reinterpret_cast<const f32x4 *>(x + i);
         if (splits > 0) {
-            float p = part[i];
-            for (int s = 1; s < splits; s++) p = __fadd_rn(p, part[(size_t)s * part_stride + i]);
-            a = __fadd_rn(a, p);
-            x[i] = a;
+            f32x4 p = *reinterpret_cast<const f32x4 *>(part + i);
+            for (int s = 1; s < splits; s++) {
+                const f32x4 q = *reinterpret_cast<const f32x4 *>(part + (size_t)s * part_stride + i);
+                p.x = __fadd_rn(p.x, q.x); p.y = __fadd_rn(p.y, q.y);
+                p.z = __fadd_rn(p.z, q.z); p.w = __fadd_rn(p.w, q.w);
+            }
+            a.x = __fadd_rn(a.x, p.x); a.y = __fadd_rn(a.y, p.y);
+            a.z = __fadd_rn(a.z, p.z); a.w = __fadd_rn(a.w, p.w);
+            *reinterpret_cast<f32x4 *>(x + i) = a;
         }
         v[j] = a;
-        ss = fmaf(a, a, ss);
+        ss = fmaf(a.x, a.x, ss); ss = fmaf(a.y, a.y, ss);
+        ss = fmaf(a.z, a.z, ss); ss = fmaf(a.w, a.w, ss);
     }
     if (!w) return;
     ss = vt_wave_sum(ss);
@@ -230,12 +239,16 @@ vt_residual_norm_split_kernel(float *x, const float *part, int splits, size_t pa
     const float tot = (red[0] + red[1]) + (red[2] + red[3]);
     const float inv = 1.0f / sqrtf(tot / (float)VT_DIM + eps);
 #pragma unroll
-    for (int j = 0; j < VT_DIM / 256; j++) {
-        const int c = (int)threadIdx.x + 256 * j;
-        unsigned h, l;
-        vt_split_planes(__fmul_rn(__fmul_rn(v[j], inv), w[c]), h, l);
-        hi[row * VT_DIM + c] = (uint16_t)h;
-        lo[row * VT_DIM + c] = (uint16_t)l;
+    for (int j = 0; j < NJ; j++) {
+        const int c = 4 * ((int)threadIdx.x + 256 * j);
+        const f32x4 g = *reinterpret_cast<const f32x4 *>(w + c);
+        unsigned h0, l0, h1, l1, h2, l2, h3, l3;
+        vt_split_planes(__fmul_rn(__fmul_rn(v[j].x, inv), g.x), h0, l0);
+        vt_split_planes(__fmul_rn(__fmul_rn(v[j].y, inv), g.y), h1, l1);
+        vt_split_planes(__fmul_rn(__fmul_rn(v[j].z, inv), g.z), h2, l2);
+        vt_split_planes(__fmul_rn(__fmul_rn(v[j].w, inv), g.w), h3, l3);
+        *reinterpret_cast<u32x2 *>(hi + row * VT_DIM + c) = u32x2{h0 | (h1 << 16), h2 | (h3 << 16)};
+        *reinterpret_cast<u32x2 *>(lo + row * VT_DIM + c) = u32x2{l0 | (l1 << 16), l2 | (l3 << 16)};
     }
 }
 
@@ -249,39 +262,50 @@ void vt_launch_residual_norm_split(float *d_x, const float *d_part, int splits, 
  * (voxtral_tts_llm.c:346-350 on the row-interleaved gate/up matrix).  Columns from
  * tail_col0 on are taken as the sum of `tail_planes` split-K planes [rows, 2*ffn - tail_col0]
  * instead (tail_planes == 0: everything is in gu). */
-__global__ void vt_swiglu_split_kernel(uint16_t *hi, uint16_t *lo, const float *gu, size_t n2,
+__global__ void vt_swiglu_split_kernel(uint16_t *hi, uint16_t *lo, const float *gu, size_t n8,
                                        int tail_col0, const float *tail, int tail_planes, size_t tail_stride) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n2;
+    /* a thread owns 8 consecutive floats, i.e. 4 (gate, up) pairs: 16-byte loads, 8-byte plane
+     * stores; rows and the tail boundary are multiples of 8 columns */
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
          i += (size_t)gridDim.x * blockDim.x) {
-        f32x4 g = reinterpret_cast<const f32x4 *>(gu)[i];
+        f32x4 g0 = reinterpret_cast<const f32x4 *>(gu)[2 * i];
+        f32x4 g1 = reinterpret_cast<const f32x4 *>(gu)[2 * i + 1];
         if (tail_planes > 0) {
-            const size_t row = (4 * i) / (2 * VT_FFN);
-            const int col = (int)((4 * i) % (2 * VT_FFN));
+            const size_t row = (8 * i) / (2 * VT_FFN);
+            const int col = (int)((8 * i) % (2 * VT_FFN));
             if (col >= tail_col0) {
                 const int tw = 2 * VT_FFN - tail_col0;
                 const float *tp = tail + row * tw + (col - tail_col0);
-                g = *reinterpret_cast<const f32x4 *>(tp);
+                g0 = *reinterpret_cast<const f32x4 *>(tp);
+                g1 = *reinterpret_cast<const f32x4 *>(tp + 4);
                 for (int p = 1; p < tail_planes; p++) {
-                    const f32x4 w = *reinterpret_cast<const f32x4 *>(tp + p * tail_stride);
-                    g.x = __fadd_rn(g.x, w.x); g.y = __fadd_rn(g.y, w.y);
-                    g.z = __fadd_rn(g.z, w.z); g.w = __fadd_rn(g.w, w.w);
+                    const f32x4 w0 = *reinterpret_cast<const f32x4 *>(tp + p * tail_stride);
+                    const f32x4 w1 = *reinterpret_cast<const f32x4 *>(tp + p * tail_stride + 4);
+                    g0.x = __fadd_rn(g0.x, w0.x); g0.y = __fadd_rn(g0.y, w0.y);
+                    g0.z = __fadd_rn(g0.z, w0.z); g0.w = __fadd_rn(g0.w, w0.w);
+                    g1.x = __fadd_rn(g1.x, w1.x); g1.y = __fadd_rn(g1.y, w1.y);
+                    g1.z = __fadd_rn(g1.z, w1.z); g1.w = __fadd_rn(g1.w, w1.w);
                 }
             }
         }
-        const float a = __fmul_rn(__fdiv_rn(g.x, __fadd_rn(1.0f, expf(-g.x))), g.y);
-        const float b = __fmul_rn(__fdiv_rn(g.z, __fadd_rn(1.0f, expf(-g.z))), g.w);
-        unsigned h0, l0, h1, l1;
+        const float a = __fmul_rn(__fdiv_rn(g0.x, __fadd_rn(1.0f, expf(-g0.x))), g0.y);
+        const float b = __fmul_rn(__fdiv_rn(g0.z, __fadd_rn(1.0f, expf(-g0.z))), g0.w);
+        const float c = __fmul_rn(__fdiv_rn(g1.x, __fadd_rn(1.0f, expf(-g1.x))), g1.y);
+        const float d = __fmul_rn(__fdiv_rn(g1.z, __fadd_rn(1.0f, expf(-g1.z))), g1.w);
+        unsigned h0, l0, h1, l1, h2, l2, h3, l3;
         vt_split_planes(a, h0, l0);
         vt_split_planes(b, h1, l1);
-        reinterpret_cast<unsigned *>(hi)[i] = h0 | (h1 << 16);
-        reinterpret_cast<unsigned *>(lo)[i] = l0 | (l1 << 16);
+        vt_split_planes(c, h2, l2);
+        vt_split_planes(d, h3, l3);
+        reinterpret_cast<u32x2 *>(hi)[i] = u32x2{h0 | (h1 << 16), h2 | (h3 << 16)};
+        reinterpret_cast<u32x2 *>(lo)[i] = u32x2{l0 | (l1 << 16), l2 | (l3 << 16)};
     }
 }
 
 void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, size_t n_out, int tail_col0,
                             const float *d_tail, int tail_planes, size_t tail_stride) {
-    hipLaunchKernelGGL(vt_swiglu_split_kernel, dim3(gm_blocks(n_out / 2)), dim3(256), 0, g_vt.stream, d_hi, d_lo,
-                       d_gu, n_out / 2, tail_col0, d_tail, tail_planes, tail_stride);
+    hipLaunchKernelGGL(vt_swiglu_split_kernel, dim3(gm_blocks(n_out / 4)), dim3(256), 0, g_vt.stream, d_hi, d_lo,
+                       d_gu, n_out / 4, tail_col0, d_tail, tail_planes, tail_stride);
 }
 
 /* C = sum of `splits` partial planes (fixed order), for callers that want the plain product. */

@@ -21,31 +21,33 @@
  * q [S,4096] with RoPE, cache rows start_pos.. (k with RoPE, v) */
 __global__ void vt_split_qkv_rope_kernel(const float *qkv, int planes, size_t plane_stride, float *q,
                                          float *kc, float *vc, const float *rope, int start_pos, int S) {
-    const int pairs = VT_QKV_DIM / 2;
-    const size_t total = (size_t)S * pairs;
+    /* a thread owns two adjacent RoPE pairs: 16-byte loads and stores */
+    const int quads = VT_QKV_DIM / 4;
+    const size_t total = (size_t)S * quads;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (size_t)gridDim.x * blockDim.x) {
-        const int s = (int)(i / pairs), g = (int)(i % pairs) * 2;
-        f32x2 ab = *reinterpret_cast<const f32x2 *>(qkv + (size_t)s * VT_QKV_DIM + g);
+        const int s = (int)(i / quads), g = (int)(i % quads) * 4;
+        f32x4 ab = *reinterpret_cast<const f32x4 *>(qkv + (size_t)s * VT_QKV_DIM + g);
         for (int p = 1; p < planes; p++) {
-            const f32x2 w = *reinterpret_cast<const f32x2 *>(qkv + p * plane_stride + (size_t)s * VT_QKV_DIM + g);
-            ab.x = __fadd_rn(ab.x, w.x);
-            ab.y = __fadd_rn(ab.y, w.y);
+            const f32x4 w = *reinterpret_cast<const f32x4 *>(qkv + p * plane_stride + (size_t)s * VT_QKV_DIM + g);
+            ab.x = __fadd_rn(ab.x, w.x); ab.y = __fadd_rn(ab.y, w.y);
+            ab.z = __fadd_rn(ab.z, w.z); ab.w = __fadd_rn(ab.w, w.w);
         }
-        f32x2 o = ab;
+        f32x4 o = ab;
         float *dst;
         if (g < VT_Q_DIM + VT_KV_DIM) {
-            const float *cs = rope + (size_t)(start_pos + s) * VT_HEAD_DIM;
-            const int d = (g & (VT_HEAD_DIM - 1)) >> 1;
-            const float c = cs[2 * d], sn = cs[2 * d + 1];
-            o.x = __fsub_rn(__fmul_rn(ab.x, c), __fmul_rn(ab.y, sn));
-            o.y = __fadd_rn(__fmul_rn(ab.x, sn), __fmul_rn(ab.y, c));
+            const int d = (g & (VT_HEAD_DIM - 1)) >> 1;         /* first of the two pairs */
+            const f32x4 cs = *reinterpret_cast<const f32x4 *>(rope + (size_t)(start_pos + s) * VT_HEAD_DIM + 2 * d);
+            o.x = __fsub_rn(__fmul_rn(ab.x, cs.x), __fmul_rn(ab.y, cs.y));
+            o.y = __fadd_rn(__fmul_rn(ab.x, cs.y), __fmul_rn(ab.y, cs.x));
+            o.z = __fsub_rn(__fmul_rn(ab.z, cs.z), __fmul_rn(ab.w, cs.w));
+            o.w = __fadd_rn(__fmul_rn(ab.z, cs.w), __fmul_rn(ab.w, cs.z));
             dst = g < VT_Q_DIM ? q + (size_t)s * VT_Q_DIM + g
                                : kc + (size_t)(start_pos + s) * VT_KV_DIM + (g - VT_Q_DIM);
         } else {
             dst = vc + (size_t)(start_pos + s) * VT_KV_DIM + (g - VT_Q_DIM - VT_KV_DIM);
         }
-        *reinterpret_cast<f32x2 *>(dst) = o;
+        *reinterpret_cast<f32x4 *>(dst) = o;
     }
 }
 
@@ -316,7 +318,7 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         float *kc = g_hip.kv_cache_k_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
         float *vc = g_hip.kv_cache_v_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
         vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
-        hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(ew_blocks(S * VT_QKV_DIM / 2)), dim3(256), 0, st,
+        hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(ew_blocks(S * VT_QKV_DIM / 4)), dim3(256), 0, st,
                            wide, sp_qkv, S * VT_QKV_DIM, q, kc, vc, g_vt.d_rope, start_pos, seq_len);
         vt_launch_prefill_attention(NULL, hi, lo, q, VT_Q_DIM, kc, vc, seq_len, start_pos);
         vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
