@@ -278,9 +278,11 @@ void tts_hip_timer_start(void);
 float tts_hip_timer_stop_ms(void);
 /* Average duration in ms of one launch of a single kernel, timed with events on the
  * internal stream over `iters` launches on zero-filled work buffers (needs the weights
- * of layer 0 uploaded): which 0..3 = sequence-level product at M = 512 with the q|k|v,
- * output, gate/up and down projection; 4 = causal attention at 512 queries (KV cache of
- * at least 512 rows); 10..13 = the four acoustic phase kernels; 20..23 = the codec's fp32
+ * uploaded; launch i takes the weights of uploaded layer i modulo their number, so that they
+ * come from HBM as in a real pass): which 0..3 = sequence-level product at M = 512 with the
+ * q|k|v, output, gate/up and down projection; 4 = causal attention at 512 queries (KV cache
+ * of at least 512 rows); 10..13 = the four acoustic phase kernels, 14 = the four of them in
+ * order on one layer (the value is the duration of all four); 20..23 = the codec's fp32
  * product at 1600 rows with the q|k|v, output, gate|up and down matrices, 24 = the whole codec
  * decoder on 200 frames (codec weights uploaded).  Negative on error. */
 float tts_hip_bench_kernel(int which, int iters);

@@ -350,20 +350,21 @@ extern "C" void tts_hip_llm_prefill(const float *embeds, int seq_len, int start_
 
 /* ---- single-kernel timing for benchmarks ---------------------------------------------
  * which 0..3: the matrix-core product at M = 512 with the q|k|v, output, gate/up and
- * down projection of backbone layer 0 (splits as in the prefill); 4: the causal
- * attention at 512 queries; 10..13: the four acoustic phase kernels of acoustic layer 0.
+ * down projection (splits as in the prefill), every launch on the next backbone layer's
+ * weights; 4: the causal attention at 512 queries; 10..13: the four acoustic phase kernels,
+ * every launch on the next acoustic layer; 14: the four phase launches of one acoustic layer
+ * in order (the value is the time of all four).
  * Returns the average duration of one launch in ms (events on the internal stream), or
  * a negative value on error.  Buffers hold zeros: the kernels are data-independent. */
 float vt_bench_acoustic_phase(int phase, int iters);
 
 extern "C" float tts_hip_bench_kernel(int which, int iters) {
     if (!g_vt.initialized || iters < 1) { vt_set_error("tts_hip_bench_kernel: bad call"); return -1.f; }
-    if (which >= 10 && which <= 13) return vt_bench_acoustic_phase(which - 10, iters);
+    if (which >= 10 && which <= 14) return vt_bench_acoustic_phase(which - 10, iters);
     if (which >= 20 && which <= 24) return vt_bench_codec(which - 20, iters);
     if (which < 0 || which > 4 || g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_bench_kernel: unknown kernel %d", which); return -1.f; }
     const int S = 512;
     if (which == 4 && g_vt.kv_max < S) { vt_set_error("tts_hip_bench_kernel: KV cache shorter than 512"); return -1.f; }
-    const vt_layer_dev *L = &g_vt.h_layers[0];
     static const int NN[4] = {VT_QKV_DIM, VT_DIM, 2 * VT_FFN, VT_DIM}, KK[4] = {VT_DIM, VT_Q_DIM, VT_DIM, VT_FFN},
                      SP[4] = {2, 4, 1, 4};
     const size_t n_out = (size_t)S * 2 * VT_FFN * 4, n_plane = (size_t)S * VT_FFN, n_q = (size_t)S * VT_Q_DIM;
@@ -373,10 +374,13 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
     if (vt_check(hipMemsetAsync(base, 0, bytes, g_vt.stream), "bench clear")) return -1.f;
     float *out = (float *)base, *q = out + n_out;
     uint16_t *hi = (uint16_t *)(q + n_q), *lo = hi + n_plane;
-    const uint16_t *W[4] = {L->wqkv, L->wo, L->w13, L->w2};
     float ms = -1.f;
     for (int it = -2; it < iters; it++) {
         if (it == 0 && vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench start")) return -1.f;
+        /* every launch takes the next layer's weights, as in a prefill: launched again and again on
+         * one layer they would be served from the memory-side cache */
+        const vt_layer_dev *L = &g_vt.h_layers[(it + 2) % g_vt.n_dec_layers];
+        const uint16_t *W[4] = {L->wqkv, L->wo, L->w13, L->w2};
         if (which == 2) {                               /* as in the prefill: main part + K-cut tail */
             const int tail = 16 * 128, main_cols = 2 * VT_FFN - tail;
             vt_launch_gemm_ex(out, 2 * VT_FFN, 0, hi, lo, W[2], S, main_cols, VT_DIM, 1);
