@@ -153,3 +153,29 @@ def test_end_audio_frame(ac_session):
     codes, x = hip.acoustic_frame(S.f32_normal(S.DIM, 30), np.zeros(S.ACOUSTIC_DIM, np.float32))
     assert codes[0] == 1 and np.all(codes[1:] == 2)
     hip.upload_acoustic(ac)
+
+
+def test_single_kernel_timing_modes(ac_session):
+    """The event-timed launches bench.py prices its roofline on: each acoustic phase
+    alone (10..13) and the four of a layer in order (14) return a positive time, the
+    in-order figure lies between the largest phase and a generous multiple of their
+    sum, and an unknown selector is an error, not a launch."""
+    hip, orc, ac = ac_session
+    alone = [hip.lib.tts_hip_bench_kernel(w, 5) for w in (10, 11, 12, 13)]
+    layer = hip.lib.tts_hip_bench_kernel(14, 5)
+    hip.check()
+    assert all(0.0 < a < 1.0 for a in alone), alone
+    assert max(alone) < layer < 3.0 * sum(alone), (alone, layer)
+    n0 = hip.lib.tts_hip_error_count()
+    assert hip.lib.tts_hip_bench_kernel(15, 5) < 0
+    assert hip.lib.tts_hip_bench_kernel(14, 0) < 0
+    assert hip.lib.tts_hip_error_count() == n0 + 2
+    hip.err0 = n0 + 2                                      # the two errors above were asked for
+    # the frame still runs after the timing loops used the same work buffers
+    gold = np.load(os.path.join(S.GOLDEN_DIR, "acoustic.npz"))
+    st = C.c_uint64(0)
+    S.oracle().orc_rng_seed(C.byref(st), 42)
+    x0 = np.zeros(S.ACOUSTIC_DIM, np.float32)
+    S.oracle().orc_randn_fill(C.byref(st), S.fp(x0), S.ACOUSTIC_DIM)
+    codes, _ = hip.acoustic_frame(S.f32_normal(S.DIM, 20), x0)
+    assert np.array_equal(codes, gold["codes"][0])
