@@ -238,7 +238,7 @@ __device__ __forceinline__ void ac_consume(const u32x4 (&wreg)[NL], const unsign
 /* cross-wave sum of one unit and its epilogue; `red` is this unit's buffer */
 template <int PH>
 __device__ __forceinline__ void ac_finish_unit(const ac_phase_args &a, float *red, int n0, f32x4 acc_hi,
-                                               f32x4 acc_lo) {
+                                               f32x4 acc_lo, bool have_prev = false, float prev = 0.f) {
     const int lane = vt_lane(), wave = vt_wave(), col = lane & 15, kg = lane >> 4;
     /* accumulator element v of lane l: activation row 4*(l/16) + v, weight row l%16 */
 #pragma unroll
@@ -268,7 +268,7 @@ __device__ __forceinline__ void ac_finish_unit(const ac_phase_args &a, float *re
             a.out[(size_t)m * VT_QKV_DIM + n0 + n] = y;
         } else {
             float *p = a.out + (size_t)m * VT_DIM + n0 + n;
-            *p = __fadd_rn(*p, y);
+            *p = __fadd_rn(have_prev ? prev : *p, y);
         }
     }
 }
@@ -296,6 +296,16 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
     const unsigned char *fl = lo + arow * SH::PITCH + 2 * (wave * SH::KW + 8 * kg);
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     u32x4 w0[SH::NL], w1[SH::NL];
+    /* the residual this workgroup's first unit is added to is requested before everything else (a
+     * load of its own at the end of the kernel would cost a round trip to memory after the last
+     * product); every thread asks, the ones without an output element for element 0 */
+    const int first_unit = u;
+    float prev = 0.f;
+    if (PH == AC_WO || PH == AC_W2) {
+        const int t = (int)threadIdx.x;
+        const bool fin = t < AC_ROWS * 16 && (t & 15) < AC_RB;
+        prev = a.out[(size_t)(fin ? t >> 4 : 0) * VT_DIM + u * AC_RB + (fin ? t & 15 : 0)];
+    }
 
     if (SH::NPASS == 1) {
         ac_rows_regs rr;
@@ -315,7 +325,7 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
             if (nx >= n_units) {
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w0, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al);
+                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
                 break;
             }
             {
@@ -323,14 +333,14 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
                 __builtin_amdgcn_sched_barrier(0);
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w0, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al);
+                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
                 u = nx;
             }
             nx = u + G;
             if (nx >= n_units) {
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w1, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al);
+                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
                 break;
             }
             {
@@ -338,7 +348,7 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
                 __builtin_amdgcn_sched_barrier(0);
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w1, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al);
+                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
                 u = nx;
             }
         }
@@ -361,7 +371,7 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
                 }
                 ac_consume(wreg[pass & 1], fa, fl, ah, al);
             }
-            ac_finish_unit<PH>(a, red, u * AC_RB, ah, al);
+            ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
         }
     }
 }
