@@ -58,14 +58,17 @@ template <int PH> struct ac_shape {
     static constexpr int NL = KW / 32;                               /* 16-byte loads per lane and pass */
     static constexpr int PITCH = KP * 2 + 16;                        /* bytes per plane row */
     static constexpr int PLANE = AC_ROWS * PITCH;
-    static constexpr int LDS_BYTES = 2 * PLANE + 4 * (2 * AC_WAVES * AC_ROWS * 16 + AC_WAVES * 8);
+    static constexpr int RED_BYTES = 4 * (2 * AC_WAVES * AC_ROWS * 16 + AC_WAVES * 8);
+    /* attention + output projection: the k|v columns of the 6 rows, shared by the 4 heads of a group */
+    static constexpr int KV_BYTES = PH == AC_WO ? AC_ROWS * 2 * VT_KV_DIM * 4 : 0;
+    static constexpr int LDS_BYTES = 2 * PLANE + RED_BYTES + KV_BYTES;
 };
 
 /* Activation rows are fetched into registers BEFORE the weight loads of a pass are
  * issued: a wave's loads return in order, so this way the planes can be built while
  * the weights are still streaming in. */
 struct ac_rows_regs { f32x4 v[AC_ROWS][2]; f32x4 g[2]; };
-struct ac_attn_regs { f32x4 q[3][4], k[3][4], v[3][4]; };
+struct ac_attn_regs { f32x4 q[3][4]; f32x4 kv[AC_ROWS * 2 * VT_KV_DIM / 4 / AC_THREADS]; };
 
 /* rows of 3072 = 768 groups of 4 columns: thread t owns group t, and group 512 + t when t < 256
  * (16-byte loads: half the load instructions of 8-byte ones for the same bytes) */
@@ -145,27 +148,49 @@ __device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned ch
 
 /* Bidirectional attention over the 3 tokens of each branch, straight into the
  * planes that feed the output projection (tts_bidirectional_attention,
- * voxtral_tts_kernels.c:467-525).  8 lanes per (branch, head), 16 dims each. */
+ * voxtral_tts_kernels.c:467-525).  8 lanes per (branch, head), 16 dims each.  Every
+ * lane keeps its q in registers; k and v, which the 4 heads of a group share, are
+ * fetched once per workgroup (k|v are 2048 consecutive floats of a row) and handed
+ * round through LDS: each head fetching its own copy made this kernel pull 295 KB
+ * of activations through its CU instead of 147 KB. */
 __device__ __forceinline__ void ac_fetch_attn(ac_attn_regs &r, const float *qkv) {
     const int lane = vt_lane(), pair = vt_wave() * 8 + (lane >> 3), sub = lane & 7;
     const int br = pair >> 5, h = pair & 31, d0 = sub * 16;
+    constexpr int ROW4 = 2 * VT_KV_DIM / 4;                    /* 16-byte groups of k|v per row */
+#pragma unroll
+    for (int j = 0; j < AC_ROWS * ROW4 / AC_THREADS; j++) {
+        const int i = (int)threadIdx.x + AC_THREADS * j;
+        r.kv[j] = *reinterpret_cast<const f32x4 *>(qkv + (size_t)(i / ROW4) * VT_QKV_DIM + VT_Q_DIM + 4 * (i % ROW4));
+    }
 #pragma unroll
     for (int i = 0; i < 3; i++) {
         const float *row = qkv + (size_t)(br * 3 + i) * VT_QKV_DIM;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            r.q[i][e] = *reinterpret_cast<const f32x4 *>(row + h * VT_HEAD_DIM + d0 + 4 * e);
-            r.k[i][e] = *reinterpret_cast<const f32x4 *>(row + VT_Q_DIM + (h >> 2) * VT_HEAD_DIM + d0 + 4 * e);
-            r.v[i][e] = *reinterpret_cast<const f32x4 *>(row + VT_Q_DIM + VT_KV_DIM + (h >> 2) * VT_HEAD_DIM + d0 + 4 * e);
-        }
+        for (int e = 0; e < 4; e++) r.q[i][e] = *reinterpret_cast<const f32x4 *>(row + h * VT_HEAD_DIM + d0 + 4 * e);
     }
 }
 
+/* k|v of the 6 rows into LDS as [row][2048] */
+__device__ __forceinline__ void ac_stage_kv(f32x4 *kvl, const ac_attn_regs &r) {
+#pragma unroll
+    for (int j = 0; j < AC_ROWS * 2 * VT_KV_DIM / 4 / AC_THREADS; j++) kvl[(int)threadIdx.x + AC_THREADS * j] = r.kv[j];
+}
+
 __device__ __forceinline__ void ac_attention_to_planes(unsigned char *hi, unsigned char *lo, int pitch,
-                                                       const ac_attn_regs &r) {
+                                                       const ac_attn_regs &r, const f32x4 *kvl) {
     const int lane = vt_lane(), pair = vt_wave() * 8 + (lane >> 3), sub = lane & 7;
     const int br = pair >> 5, h = pair & 31, d0 = sub * 16;
     const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
+    constexpr int ROW4 = 2 * VT_KV_DIM / 4;
+    f32x4 k[3][4], v[3][4];
+#pragma unroll
+    for (int j = 0; j < 3; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int at = (br * 3 + j) * ROW4 + ((h >> 2) * VT_HEAD_DIM + d0) / 4 + e;
+            k[j][e] = kvl[at];
+            v[j][e] = kvl[at + VT_KV_DIM / 4];
+        }
 #pragma unroll
     for (int i = 0; i < 3; i++) {
         float s[3];
@@ -174,10 +199,10 @@ __device__ __forceinline__ void ac_attention_to_planes(unsigned char *hi, unsign
             float p = 0.f;
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                p = fmaf(r.q[i][e].x, r.k[j][e].x, p);
-                p = fmaf(r.q[i][e].y, r.k[j][e].y, p);
-                p = fmaf(r.q[i][e].z, r.k[j][e].z, p);
-                p = fmaf(r.q[i][e].w, r.k[j][e].w, p);
+                p = fmaf(r.q[i][e].x, k[j][e].x, p);
+                p = fmaf(r.q[i][e].y, k[j][e].y, p);
+                p = fmaf(r.q[i][e].z, k[j][e].z, p);
+                p = fmaf(r.q[i][e].w, k[j][e].w, p);
             }
             p += vt_dpp<0xB1>(p);                 /* lanes ^1 */
             p += vt_dpp<0x4E>(p);                 /* lanes ^2 */
@@ -191,10 +216,10 @@ __device__ __forceinline__ void ac_attention_to_planes(unsigned char *hi, unsign
         unsigned char *pl = lo + (br * 3 + i) * pitch + 2 * (h * VT_HEAD_DIM + d0);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const float o0 = __fmul_rn(fmaf(p2, r.v[2][e].x, fmaf(p1, r.v[1][e].x, p0 * r.v[0][e].x)), inv);
-            const float o1 = __fmul_rn(fmaf(p2, r.v[2][e].y, fmaf(p1, r.v[1][e].y, p0 * r.v[0][e].y)), inv);
-            const float o2 = __fmul_rn(fmaf(p2, r.v[2][e].z, fmaf(p1, r.v[1][e].z, p0 * r.v[0][e].z)), inv);
-            const float o3 = __fmul_rn(fmaf(p2, r.v[2][e].w, fmaf(p1, r.v[1][e].w, p0 * r.v[0][e].w)), inv);
+            const float o0 = __fmul_rn(fmaf(p2, v[2][e].x, fmaf(p1, v[1][e].x, p0 * v[0][e].x)), inv);
+            const float o1 = __fmul_rn(fmaf(p2, v[2][e].y, fmaf(p1, v[1][e].y, p0 * v[0][e].y)), inv);
+            const float o2 = __fmul_rn(fmaf(p2, v[2][e].z, fmaf(p1, v[1][e].z, p0 * v[0][e].z)), inv);
+            const float o3 = __fmul_rn(fmaf(p2, v[2][e].w, fmaf(p1, v[1][e].w, p0 * v[0][e].w)), inv);
             unsigned h0, l0, h1, l1, h2, l2, h3, l3;
             vt_split_planes(o0, h0, l0);
             vt_split_planes(o1, h1, l1);
@@ -312,8 +337,12 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
         ac_attn_regs ra;
         if (PH == AC_WO) ac_fetch_attn(ra, a.in); else ac_fetch_rows(rr, a.in, VT_DIM, a.gain);
         ac_issue<PH>(w0, wbase + u * unit_stride);
-        if (PH == AC_WO) ac_attention_to_planes(hi, lo, SH::PITCH, ra);
-        else ac_rows_to_planes<true>(hi, lo, SH::PITCH, rr, red_ss);
+        if (PH == AC_WO) {
+            f32x4 *kvl = reinterpret_cast<f32x4 *>(ac_lds + 2 * SH::PLANE + SH::RED_BYTES);
+            ac_stage_kv(kvl, ra);
+            __syncthreads();
+            ac_attention_to_planes(hi, lo, SH::PITCH, ra, kvl);
+        } else ac_rows_to_planes<true>(hi, lo, SH::PITCH, rr, red_ss);
         __syncthreads();
         /* The request for unit u + G is never issued under a condition of its own: the compiler
          * counts outstanding loads statically, and behind a conditional request it would make the
