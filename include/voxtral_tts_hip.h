@@ -293,6 +293,13 @@ float tts_hip_bench_kernel(int which, int iters);
  * Negative on error. */
 float tts_hip_bench_matvec(float *d_y, const float *d_x, const uint16_t *d_W, size_t copy_stride,
                            int n_copies, int in_dim, int out_dim, int iters);
+/* The activation format of the sequence-level products: n fp32 values (n even, device pointers,
+ * 8-byte aligned) -> two bf16 planes, hi = bf16(x) rounded to nearest even and lo = bf16(x - hi),
+ * so that hi + lo carries x to about 2^-17 relative (tts_hip_linear_bf16 with seq_len >= 8 and
+ * tts_hip_llm_prefill multiply every weight tile with both planes).  No counterpart in the
+ * reference, whose CPU products read the fp32 activations directly (voxtral_tts_kernels.c:127-138);
+ * exported so that the format can be checked bit for bit.  Returns 0, or -1 on error. */
+int tts_hip_split_planes(uint16_t *d_hi, uint16_t *d_lo, const float *d_x, size_t n);
 
 #ifdef __cplusplus
 }

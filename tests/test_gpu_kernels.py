@@ -194,6 +194,59 @@ def test_embed_token_exact(hip, orc):
     assert np.array_equal(do.to_numpy(np.float32, S.DIM), orc.embed_token(emb, 33))
 
 
+def _bf16_rne(x):
+    """bf16 bits of fp32 values, round to nearest even, in integer arithmetic (finite inputs)."""
+    u = x.view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def test_split_planes_bit_exact(hip):
+    """hi = bf16(x), lo = bf16(x - hi) with round to nearest even: the device uses the
+    packed hardware conversion, the model here is integer arithmetic.  Random values over
+    many magnitudes, exact ties in both directions, values that round up into the next
+    binade, zeros of both signs, the largest finite value bf16 does not round to
+    infinity, and residuals that fall into the fp32 denormal range."""
+    rng = np.random.default_rng(5)
+    parts = [
+        (rng.standard_normal(1 << 16) * np.exp(rng.uniform(-20, 20, 1 << 16))).astype(np.float32),
+        # ties: low half exactly 0x8000 with even and odd bf16 mantissas, and just around them
+        np.array([0x3F808000, 0x3F818000, 0x3F807FFF, 0x3F808001, 0xBF808000, 0xBF818000,
+                  0x3FFF8000, 0x3FFFFFFF, 0x7F7F7FFF, 0x00000000, 0x80000000,
+                  0x00810000, 0x00808000, 0x00FF8000, 0x01000001, 0x0C000001], np.uint32).view(np.float32),
+        np.float32(1.0) + np.arange(1 << 12, dtype=np.float32) * np.float32(2.0 ** -20),
+    ]
+    x = np.concatenate(parts)
+    if x.size & 1:
+        x = x[:-1]
+    d_x = dev(hip, x)
+    d_hi = H.DevBuf(hip.lib, 2 * x.size)
+    d_lo = H.DevBuf(hip.lib, 2 * x.size)
+    assert hip.lib.tts_hip_split_planes(d_hi.ptr, d_lo.ptr, d_x.ptr, x.size) == 0
+    hip.lib.tts_hip_sync()
+    hip.check()
+    hi = d_hi.to_numpy(np.uint16, x.shape)
+    lo = d_lo.to_numpy(np.uint16, x.shape)
+    want_hi = _bf16_rne(x)
+    hi_f = (want_hi.astype(np.uint32) << 16).view(np.float32)
+    resid = x - hi_f                                          # exact in fp32
+    want_lo = _bf16_rne(resid)
+    assert np.array_equal(hi, want_hi), np.flatnonzero(hi != want_hi)[:8]
+    bad = np.flatnonzero(lo != want_lo)
+    assert bad.size == 0, (bad[:8], x[bad[:8]].view(np.uint32), lo[bad[:8]], want_lo[bad[:8]])
+    # hi + lo carries x to 2^-16 of its magnitude or better
+    back = hi_f.astype(np.float64) + (lo.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    big = np.abs(x) > 1e-30
+    assert np.max(np.abs(back[big] - x[big]) / np.abs(x[big])) < 2.0 ** -16
+    # an odd count and a misaligned pointer are refused
+    n0 = hip.lib.tts_hip_error_count()
+    assert hip.lib.tts_hip_split_planes(d_hi.ptr, d_lo.ptr, d_x.ptr, 3) == -1
+    assert hip.lib.tts_hip_split_planes(d_hi.ptr, d_lo.ptr, d_x.ptr + 4, 2) == -1
+    assert hip.lib.tts_hip_error_count() == n0 + 2
+    hip.err0 = n0 + 2
+    for b in (d_x, d_hi, d_lo):
+        b.free()
+
+
 def test_bad_arguments_are_reported_not_executed(hip):
     n0 = hip.lib.tts_hip_error_count()
     hip.lib.tts_hip_rms_norm(None, None, None, 0, S.DIM, S.EPS)

@@ -117,6 +117,7 @@ SIGNATURES = {
     "tts_hip_timer_stop_ms": (C.c_float, []),
     "tts_hip_bench_kernel": (C.c_float, [C.c_int, C.c_int]),
     "tts_hip_bench_matvec": (C.c_float, [vp, vp, vp, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "tts_hip_split_planes": (C.c_int, [vp, vp, vp, C.c_size_t]),
     "tts_hip_upload_audio_embeddings": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "tts_hip_audio_embed": (None, [C.c_void_p, C.c_void_p]),
     "tts_hip_generate_frame": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]),

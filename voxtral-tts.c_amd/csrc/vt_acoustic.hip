@@ -134,13 +134,10 @@ __device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned ch
                     v.z = __fmul_rn(__fmul_rn(v.z, inv[m]), g.z);
                     v.w = __fmul_rn(__fmul_rn(v.w, inv[m]), g.w);
                 }
-                unsigned h0, l0, h1, l1, h2, l2, h3, l3;
-                vt_split_planes(v.x, h0, l0);
-                vt_split_planes(v.y, h1, l1);
-                vt_split_planes(v.z, h2, l2);
-                vt_split_planes(v.w, h3, l3);
-                *reinterpret_cast<u32x2 *>(hi + m * pitch + 2 * c) = u32x2{h0 | (h1 << 16), h2 | (h3 << 16)};
-                *reinterpret_cast<u32x2 *>(lo + m * pitch + 2 * c) = u32x2{l0 | (l1 << 16), l2 | (l3 << 16)};
+                u32x2 sph, spl;
+                vt_split_planes4(v.x, v.y, v.z, v.w, sph, spl);
+                *reinterpret_cast<u32x2 *>(hi + m * pitch + 2 * c) = sph;
+                *reinterpret_cast<u32x2 *>(lo + m * pitch + 2 * c) = spl;
             }
         }
     }
@@ -220,12 +217,9 @@ __device__ __forceinline__ void ac_attention_to_planes(unsigned char *hi, unsign
             const float o1 = __fmul_rn(fmaf(p2, v[2][e].y, fmaf(p1, v[1][e].y, p0 * v[0][e].y)), inv);
             const float o2 = __fmul_rn(fmaf(p2, v[2][e].z, fmaf(p1, v[1][e].z, p0 * v[0][e].z)), inv);
             const float o3 = __fmul_rn(fmaf(p2, v[2][e].w, fmaf(p1, v[1][e].w, p0 * v[0][e].w)), inv);
-            unsigned h0, l0, h1, l1, h2, l2, h3, l3;
-            vt_split_planes(o0, h0, l0);
-            vt_split_planes(o1, h1, l1);
-            vt_split_planes(o2, h2, l2);
-            vt_split_planes(o3, h3, l3);
-            const u32x2 vh = {h0 | (h1 << 16), h2 | (h3 << 16)}, vl = {l0 | (l1 << 16), l2 | (l3 << 16)};
+            u32x2 sph, spl;
+            vt_split_planes4(o0, o1, o2, o3, sph, spl);
+            const u32x2 vh = sph, vl = spl;
             *reinterpret_cast<u32x2 *>(ph + 8 * e) = vh;
             *reinterpret_cast<u32x2 *>(pl + 8 * e) = vl;
         }

@@ -115,9 +115,22 @@ __device__ __forceinline__ unsigned vt_bf16_rne(float x) {
     const unsigned u = __float_as_uint(x);
     return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
 }
-__device__ __forceinline__ void vt_split_planes(float x, unsigned &hi, unsigned &lo) {
-    hi = vt_bf16_rne(x);
-    lo = vt_bf16_rne(__fsub_rn(x, __uint_as_float(hi << 16)));
+/* Two values at a time, packed (first value in the low half): the vector conversion compiles to
+ * gfx950's v_cvt_pk_bf16_f32, one instruction per pair where the integer form above takes four
+ * per value; the kernels that build planes are bound by exactly these instructions. */
+typedef __bf16 vt_bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void vt_split_planes2(float a, float b, unsigned &hi, unsigned &lo) {
+    const f32x2 v = {a, b};
+    hi = __builtin_bit_cast(unsigned, __builtin_convertvector(v, vt_bf16x2));
+    const f32x2 r = {__fsub_rn(a, __uint_as_float(hi << 16)), __fsub_rn(b, __uint_as_float(hi & 0xffff0000u))};
+    lo = __builtin_bit_cast(unsigned, __builtin_convertvector(r, vt_bf16x2));
+}
+__device__ __forceinline__ void vt_split_planes4(float a, float b, float c, float d, u32x2 &hi, u32x2 &lo) {
+    unsigned h0, l0, h1, l1;
+    vt_split_planes2(a, b, h0, l0);
+    vt_split_planes2(c, d, h1, l1);
+    hi = u32x2{h0, h1};
+    lo = u32x2{l0, l1};
 }
 
 /* Device-scope coherent accesses for the small vectors that workgroups hand

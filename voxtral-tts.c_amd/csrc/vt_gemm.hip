@@ -184,11 +184,10 @@ __global__ void vt_split_kernel(uint16_t *hi, uint16_t *lo, const float *x, size
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n2;
          i += (size_t)gridDim.x * blockDim.x) {
         const f32x2 v = reinterpret_cast<const f32x2 *>(x)[i];
-        unsigned h0, l0, h1, l1;
-        vt_split_planes(v.x, h0, l0);
-        vt_split_planes(v.y, h1, l1);
-        reinterpret_cast<unsigned *>(hi)[i] = h0 | (h1 << 16);
-        reinterpret_cast<unsigned *>(lo)[i] = l0 | (l1 << 16);
+        unsigned h, l;
+        vt_split_planes2(v.x, v.y, h, l);
+        reinterpret_cast<unsigned *>(hi)[i] = h;
+        reinterpret_cast<unsigned *>(lo)[i] = l;
     }
 }
 
@@ -242,13 +241,10 @@ vt_residual_norm_split_kernel(float *x, const float *part, int splits, size_t pa
     for (int j = 0; j < NJ; j++) {
         const int c = 4 * ((int)threadIdx.x + 256 * j);
         const f32x4 g = *reinterpret_cast<const f32x4 *>(w + c);
-        unsigned h0, l0, h1, l1, h2, l2, h3, l3;
-        vt_split_planes(__fmul_rn(__fmul_rn(v[j].x, inv), g.x), h0, l0);
-        vt_split_planes(__fmul_rn(__fmul_rn(v[j].y, inv), g.y), h1, l1);
-        vt_split_planes(__fmul_rn(__fmul_rn(v[j].z, inv), g.z), h2, l2);
-        vt_split_planes(__fmul_rn(__fmul_rn(v[j].w, inv), g.w), h3, l3);
-        *reinterpret_cast<u32x2 *>(hi + row * VT_DIM + c) = u32x2{h0 | (h1 << 16), h2 | (h3 << 16)};
-        *reinterpret_cast<u32x2 *>(lo + row * VT_DIM + c) = u32x2{l0 | (l1 << 16), l2 | (l3 << 16)};
+        u32x2 sph, spl;
+        vt_split_planes4(__fmul_rn(__fmul_rn(v[j].x, inv), g.x), __fmul_rn(__fmul_rn(v[j].y, inv), g.y), __fmul_rn(__fmul_rn(v[j].z, inv), g.z), __fmul_rn(__fmul_rn(v[j].w, inv), g.w), sph, spl);
+        *reinterpret_cast<u32x2 *>(hi + row * VT_DIM + c) = sph;
+        *reinterpret_cast<u32x2 *>(lo + row * VT_DIM + c) = spl;
     }
 }
 
@@ -292,13 +288,10 @@ __global__ void vt_swiglu_split_kernel(uint16_t *hi, uint16_t *lo, const float *
         const float b = __fmul_rn(__fdiv_rn(g0.z, __fadd_rn(1.0f, expf(-g0.z))), g0.w);
         const float c = __fmul_rn(__fdiv_rn(g1.x, __fadd_rn(1.0f, expf(-g1.x))), g1.y);
         const float d = __fmul_rn(__fdiv_rn(g1.z, __fadd_rn(1.0f, expf(-g1.z))), g1.w);
-        unsigned h0, l0, h1, l1, h2, l2, h3, l3;
-        vt_split_planes(a, h0, l0);
-        vt_split_planes(b, h1, l1);
-        vt_split_planes(c, h2, l2);
-        vt_split_planes(d, h3, l3);
-        reinterpret_cast<u32x2 *>(hi)[i] = u32x2{h0 | (h1 << 16), h2 | (h3 << 16)};
-        reinterpret_cast<u32x2 *>(lo)[i] = u32x2{l0 | (l1 << 16), l2 | (l3 << 16)};
+        u32x2 sph, spl;
+        vt_split_planes4(a, b, c, d, sph, spl);
+        reinterpret_cast<u32x2 *>(hi)[i] = sph;
+        reinterpret_cast<u32x2 *>(lo)[i] = spl;
     }
 }
 

@@ -215,6 +215,17 @@ static int linear_mfma(float *d_y, const float *d_x, const uint16_t *d_W, int se
     return 1;
 }
 
+extern "C" int tts_hip_split_planes(uint16_t *d_hi, uint16_t *d_lo, const float *d_x, size_t n) {
+    if (!g_vt.initialized) { vt_set_error("tts_hip_split_planes: backend not initialised"); return -1; }
+    if (!d_hi || !d_lo || !d_x || (n & 1) || (((uintptr_t)d_x) & 7) || (((uintptr_t)d_hi | (uintptr_t)d_lo) & 3)) {
+        vt_set_error("tts_hip_split_planes: needs an even count and aligned device pointers");
+        return -1;
+    }
+    if (n == 0) return 0;
+    vt_launch_split(d_hi, d_lo, d_x, n);
+    return vt_check(hipGetLastError(), "tts_hip_split_planes") ? -1 : 0;
+}
+
 static int is_device_ptr(const void *p) {
     hipPointerAttribute_t at;
     if (hipPointerGetAttributes(&at, p) != hipSuccess) {

@@ -244,12 +244,9 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
         r.w = __fmul_rn(o[b][3], inv);
         if (out) *reinterpret_cast<f32x4 *>(out + ob + d) = r;
         if (out_hi) {
-            unsigned h0, l0, h1, l1, h2, l2, h3, l3;
-            vt_split_planes(r.x, h0, l0);
-            vt_split_planes(r.y, h1, l1);
-            vt_split_planes(r.z, h2, l2);
-            vt_split_planes(r.w, h3, l3);
-            u32x2 ph = {h0 | (h1 << 16), h2 | (h3 << 16)}, pl = {l0 | (l1 << 16), l2 | (l3 << 16)};
+            u32x2 sph, spl;
+            vt_split_planes4(r.x, r.y, r.z, r.w, sph, spl);
+            u32x2 ph = sph, pl = spl;
             *reinterpret_cast<u32x2 *>(out_hi + ob + d) = ph;
             *reinterpret_cast<u32x2 *>(out_lo + ob + d) = pl;
         }
