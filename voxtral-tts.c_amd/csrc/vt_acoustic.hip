@@ -112,13 +112,16 @@ __device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned ch
             if (vt_lane() == 0) red[vt_wave() * 8 + m] = ss;
         }
         __syncthreads();
+        /* lane m of every wave finishes row m (the division and the square root are some 50
+         * instructions; six of them in every lane were a third of this function), then the six
+         * values are broadcast from those lanes */
+        const int mrow = vt_lane() < AC_ROWS ? vt_lane() : 0;
+        float tot = 0.f;
 #pragma unroll
-        for (int m = 0; m < AC_ROWS; m++) {
-            float tot = 0.f;
+        for (int w = 0; w < AC_WAVES; w++) tot += red[w * 8 + mrow];
+        const float mine = 1.0f / sqrtf(tot / (float)VT_DIM + VT_EPS);
 #pragma unroll
-            for (int w = 0; w < AC_WAVES; w++) tot += red[w * 8 + m];
-            inv[m] = 1.0f / sqrtf(tot / (float)VT_DIM + VT_EPS);
-        }
+        for (int m = 0; m < AC_ROWS; m++) inv[m] = vt_readlane(mine, m);
     }
 #pragma unroll
     for (int j = 0; j < 2; j++) {
