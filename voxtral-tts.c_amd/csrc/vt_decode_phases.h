@@ -353,7 +353,7 @@ __device__ __forceinline__ void vt_attn_geometry(int n, int nch_max, int nw, int
  * groups keeps its own online-softmax state; they are merged through LDS at the end.  The
  * four workgroups of a kv head sit on one XCD (blockIdx % 8) and share its rows in that L2. */
 #ifndef VT_ATT_DIRECT_MAX
-#define VT_ATT_DIRECT_MAX 768      /* measured crossover with the chunked schedule (1.390 against 1.393 ms/frame at 768) */
+#define VT_ATT_DIRECT_MAX 4096     /* measured up to 4000 positions: 1.470 against 1.621 ms/frame of the chunked schedule */
 #endif
 
 /* K and V rows of one batch: 4 rounds of one position per lane group */
@@ -361,6 +361,33 @@ struct vt_att_rows { f32x4 ka[4], kb[4], va[4], vb[4]; };
 
 __device__ __forceinline__ bool vt_attn_is_direct(const vt_step_args &a) {
     return a.pos < VT_ATT_DIRECT_MAX && (int)gridDim.x >= VT_HEADS;
+}
+
+/* From a few hundred positions on, what the direct schedule costs is the K and V rows a query-head
+ * workgroup pulls through its CU (1 KB per position).  The positions of a head are then dealt to 2,
+ * 4 or 8 workgroups (every 2nd / 4th / 8th batch slot each); each leaves an un-normalised partial
+ * (max, sum, o[128]) and the output projection combines them while it stages the vector, so the
+ * phase still has no round trip of its own.  What a part costs is that combination (every
+ * workgroup of the output projection reads all partials: 16 KB per part), hence the thresholds
+ * (measured, ms/frame at 26 layers: 2 parts 1.245 against 1.263 at 400 positions, 4 parts 1.274
+ * against 1.288 at 767, 8 parts 1.283 against 1.298 at 900 and 1.470 against 1.587 at 4000). */
+#ifndef VT_ATT_SPLIT2_MIN
+#define VT_ATT_SPLIT2_MIN 384
+#endif
+#ifndef VT_ATT_SPLIT4_MIN
+#define VT_ATT_SPLIT4_MIN 656
+#endif
+#ifndef VT_ATT_SPLIT8_MIN
+#define VT_ATT_SPLIT8_MIN 896
+#endif
+#define VT_ATT_SPLIT_MAX 8
+__device__ __forceinline__ int vt_attn_split(const vt_step_args &a) {
+    if (!vt_attn_is_direct(a)) return 1;
+    const int G = (int)gridDim.x;
+    if (a.pos >= VT_ATT_SPLIT8_MIN && G >= 8 * VT_HEADS && (G & 7) == 0) return 8;
+    if (a.pos >= VT_ATT_SPLIT4_MIN && G >= 4 * VT_HEADS && (G & 7) == 0) return 4;
+    if (a.pos >= VT_ATT_SPLIT2_MIN && G >= 2 * VT_HEADS && (G & 7) == 0) return 2;
+    return 1;
 }
 
 /* Requests the rows jb, jb + stride, ... of kv head kvh (clamped to `last`; rows beyond it are
@@ -398,22 +425,24 @@ __device__ __forceinline__ void vt_attn_step(vt_att_state &st, const f32x4 &qa, 
 
 __device__ __forceinline__ void vt_attn_direct(const vt_step_args &a, int layer, float *lds) {
     const int wg = (int)blockIdx.x;
-    if (wg >= VT_HEADS) return;
-    const int kvh = wg % VT_KV_HEADS, head = kvh * 4 + wg / VT_KV_HEADS;
+    const int NS = vt_attn_split(a);
+    if (wg >= VT_HEADS * NS) return;
+    const int kvh = wg % VT_KV_HEADS, idx = wg / VT_KV_HEADS, head = kvh * 4 + (idx & 3), part_no = idx >> 2;
     const int nw = (int)(blockDim.x >> 6), wave = vt_wave(), lane = vt_lane();
     const int grp = lane >> 4, sub = lane & 15;
     const int slot = wave * 4 + grp, nslot = nw * 4;
+    const int gslot = part_no * nslot + slot, gstride = nslot * NS;     /* slot and stride over all parts */
     const int n = a.pos + 1;
     const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
     const f32x4 qa = vt_ldc4(a.q, (head * VT_HEAD_DIM + sub * 8) / 4, VT_Q_DIM);
     const f32x4 qb = vt_ldc4(a.q, (head * VT_HEAD_DIM + sub * 8) / 4 + 1, VT_Q_DIM);
     vt_att_state st = {-1e30f, 0.f, {0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    for (int jb = slot; jb < n; jb += 4 * nslot) {
+    for (int jb = gslot; jb < n; jb += 4 * gstride) {
         vt_att_rows r;
-        vt_attn_fetch(r, a, layer, kvh, jb, nslot, n - 1);
+        vt_attn_fetch(r, a, layer, kvh, jb, gstride, n - 1);
 #pragma unroll
         for (int u = 0; u < 4; u++)
-            if (jb + u * nslot < n) vt_attn_step(st, qa, qb, r.ka[u], r.kb[u], r.va[u], r.vb[u], scale);
+            if (jb + u * gstride < n) vt_attn_step(st, qa, qb, r.ka[u], r.kb[u], r.va[u], r.vb[u], scale);
     }
 
     /* merge the lane groups of the workgroup: idle slots hold (m = -1e30, l = 0, o = 0) */
@@ -428,6 +457,7 @@ __device__ __forceinline__ void vt_attn_direct(const vt_step_args &a, int layer,
         float M = vt_row16_max(ms);
         M = fmaxf(fmaxf(vt_readlane(M, 0), vt_readlane(M, 16)), fmaxf(vt_readlane(M, 32), vt_readlane(M, 48)));
         if (lane < nslot) wgt[lane] = __expf(ms - M);
+        if (lane == 0) wgt[nslot] = M;
     }
     __syncthreads();
     const int d = (int)threadIdx.x;
@@ -438,8 +468,59 @@ __device__ __forceinline__ void vt_attn_direct(const vt_step_args &a, int layer,
             Ls = fmaf(lds[w * VT_ATT_STRIDE + 1], e, Ls);
             O = fmaf(lds[w * VT_ATT_STRIDE + 4 + d], e, O);
         }
-        vt_stc(a.attn + head * VT_HEAD_DIM + d, O * (1.0f / Ls));
+        if (NS == 1) {
+            vt_stc(a.attn + head * VT_HEAD_DIM + d, O * (1.0f / Ls));
+        } else {
+            /* a part without positions leaves (max -1e30, sum 0, o 0): weight 0 in the combination */
+            float *dst = a.att_part + (size_t)(head * VT_ATT_SPLIT_MAX + part_no) * VT_ATT_STRIDE;
+            if (d == 0) { vt_stc(dst, wgt[nslot]); vt_stc(dst + 1, Ls); }
+            vt_stc(dst + 4 + d, O);
+        }
     }
+}
+
+/* The output projection's input vector into LDS: the attention output as it stands, or the
+ * combination of the NS partials per head the split schedule left (online-softmax algebra of
+ * voxtral_tts_kernels.c:426-462, parts in ascending order). */
+template <int NS>
+__device__ __forceinline__ void vt_stage_attn_parts(float *lds_x, const vt_step_args &a) {
+    f32x4 *dst = reinterpret_cast<f32x4 *>(lds_x);
+    const int total = VT_HEADS * VT_ATT_SPLIT_MAX * VT_ATT_STRIDE;
+    for (int i = (int)threadIdx.x; i < VT_Q_DIM / 4; i += (int)blockDim.x) {
+        const int head = i >> 5, d4 = i & 31;
+        const float *src = a.att_part + (size_t)head * VT_ATT_SPLIT_MAX * VT_ATT_STRIDE;
+        float m[NS], l[NS];
+        f32x4 o[NS];
+#pragma unroll
+        for (int c = 0; c < NS; c++) {
+            m[c] = vt_ldc(src + c * VT_ATT_STRIDE);
+            l[c] = vt_ldc(src + c * VT_ATT_STRIDE + 1);
+            o[c] = vt_ldc4(a.att_part, (head * VT_ATT_SPLIT_MAX + c) * (VT_ATT_STRIDE / 4) + 1 + d4, total);
+        }
+        float M = m[0];
+#pragma unroll
+        for (int c = 1; c < NS; c++) M = fmaxf(M, m[c]);
+        float Ls = 0.f;
+        f32x4 O = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < NS; c++) {
+            const float e = __expf(m[c] - M);
+            Ls = fmaf(l[c], e, Ls);
+            O.x = fmaf(o[c].x, e, O.x); O.y = fmaf(o[c].y, e, O.y);
+            O.z = fmaf(o[c].z, e, O.z); O.w = fmaf(o[c].w, e, O.w);
+        }
+        const float inv = 1.0f / Ls;
+        dst[i] = f32x4{O.x * inv, O.y * inv, O.z * inv, O.w * inv};
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ void vt_stage_attn(float *lds_x, const vt_step_args &a) {
+    const int NS = vt_attn_split(a);
+    if (NS == 8) vt_stage_attn_parts<8>(lds_x, a);
+    else if (NS == 4) vt_stage_attn_parts<4>(lds_x, a);
+    else if (NS == 2) vt_stage_attn_parts<2>(lds_x, a);
+    else vt_stage(lds_x, a.attn, VT_Q_DIM);
 }
 
 /* While a layer's attention runs on 32 workgroups, the others pull the K and V rows that the
@@ -469,7 +550,7 @@ __device__ __forceinline__ void vt_kv_l2_prefetch(const vt_step_args &a, int lay
 /* Workgroups 0 .. busy-1 run the attention of this step (busy is a multiple of 8: the same number
  * on every XCD); the others have the phase to themselves and prefetch into their L2. */
 __device__ __forceinline__ int vt_attn_busy(const vt_step_args &a) {
-    if (vt_attn_is_direct(a)) return VT_HEADS;
+    if (vt_attn_is_direct(a)) return VT_HEADS * vt_attn_split(a);
     const int nch_max = (int)gridDim.x / VT_KV_HEADS;
     int cs, nch;
     vt_attn_geometry(a.pos + 1, nch_max, (int)(blockDim.x >> 6), cs, nch);
@@ -612,7 +693,7 @@ __device__ __forceinline__ void vt_wo_body(u32x4 (&ring)[VT_RING], const vt_laye
                                            AR after_run = AR()) {
     const vt_rows r = vt_wo_rows();
     float *lds_y = lds + VT_LDS_X;
-    vt_stage(lds, a.attn, VT_Q_DIM);
+    vt_stage_attn(lds, a);
     f32x4 xa[4], xb[4];
     vt_slice_lds<4>(xa, xb, lds, r.kofs);
     /* the residual value of this thread's row, requested before any bulk load of the next phase */
