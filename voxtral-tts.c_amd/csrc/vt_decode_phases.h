@@ -364,28 +364,27 @@ __device__ __forceinline__ bool vt_attn_is_direct(const vt_step_args &a) {
 }
 
 /* From a few hundred positions on, what the direct schedule costs is the K and V rows a query-head
- * workgroup pulls through its CU (1 KB per position).  The positions of a head are then dealt to 2,
- * 4 or 8 workgroups (every 2nd / 4th / 8th batch slot each); each leaves an un-normalised partial
- * (max, sum, o[128]) and the output projection combines them while it stages the vector, so the
- * phase still has no round trip of its own.  What a part costs is that combination (every
- * workgroup of the output projection reads all partials: 16 KB per part), hence the thresholds
- * (measured, ms/frame at 26 layers: 2 parts 1.245 against 1.263 at 400 positions, 4 parts 1.274
- * against 1.288 at 767, 8 parts 1.283 against 1.298 at 900 and 1.470 against 1.587 at 4000). */
+ * workgroup pulls through its CU (1 KB per position).  The positions of a head are then dealt to 2
+ * or 8 workgroups (every 2nd / 8th batch slot each); each leaves an un-normalised partial (max,
+ * sum, o[128]) and the output projection combines them while it stages the vector, so the phase
+ * still has no round trip of its own.  What a part costs is that combination (every workgroup of
+ * the output projection reads all partials: 16 KB per part), and 8 parts take the whole grid, so
+ * that no workgroup is left to prefetch gate|up rows into L2; on the other hand 8 parts cover 1024
+ * positions in a single batch of requests.  Hence the thresholds (measured, ms/frame at 26 layers:
+ * 2 parts 1.245 against 1.263 unsplit at 400 positions; 8 parts 1.264 against 1.274 with 2 parts at
+ * 640 and 1.262 against 1.256 at 520; 4 parts were never the best: 1.274 at 640, 1.277 at 768 against
+ * 1.267 with 8; 6 parts need two batches where 8 need one: 1.376 against 1.268 at 900). */
 #ifndef VT_ATT_SPLIT2_MIN
 #define VT_ATT_SPLIT2_MIN 384
 #endif
-#ifndef VT_ATT_SPLIT4_MIN
-#define VT_ATT_SPLIT4_MIN 656
-#endif
 #ifndef VT_ATT_SPLIT8_MIN
-#define VT_ATT_SPLIT8_MIN 896
+#define VT_ATT_SPLIT8_MIN 576
 #endif
 #define VT_ATT_SPLIT_MAX 8
 __device__ __forceinline__ int vt_attn_split(const vt_step_args &a) {
     if (!vt_attn_is_direct(a)) return 1;
     const int G = (int)gridDim.x;
     if (a.pos >= VT_ATT_SPLIT8_MIN && G >= 8 * VT_HEADS && (G & 7) == 0) return 8;
-    if (a.pos >= VT_ATT_SPLIT4_MIN && G >= 4 * VT_HEADS && (G & 7) == 0) return 4;
     if (a.pos >= VT_ATT_SPLIT2_MIN && G >= 2 * VT_HEADS && (G & 7) == 0) return 2;
     return 1;
 }
@@ -518,7 +517,6 @@ __device__ __forceinline__ void vt_stage_attn_parts(float *lds_x, const vt_step_
 __device__ __forceinline__ void vt_stage_attn(float *lds_x, const vt_step_args &a) {
     const int NS = vt_attn_split(a);
     if (NS == 8) vt_stage_attn_parts<8>(lds_x, a);
-    else if (NS == 4) vt_stage_attn_parts<4>(lds_x, a);
     else if (NS == 2) vt_stage_attn_parts<2>(lds_x, a);
     else vt_stage(lds_x, a.attn, VT_Q_DIM);
 }
