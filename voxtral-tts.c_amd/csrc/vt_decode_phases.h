@@ -345,8 +345,9 @@ __device__ __forceinline__ void vt_attn_geometry(int n, int nch_max, int nw, int
     nch = (n + cs - 1) / cs;
 }
 
-/* Short caches (at most VT_ATT_DIRECT_MAX positions): one workgroup per QUERY head, no
- * cross-workgroup merge and so no store / counter / reload round trips inside the phase.
+/* Caches of fewer than VT_ATT_DIRECT_MAX positions: one workgroup per QUERY head (or several, each
+ * with a share of the positions, see vt_attn_split), no merge by a last arriver and so no
+ * store / counter / reload round trips inside the phase.
  * Lanes 16g..16g+15 of a wave serve position slot g and own 8 of the 128 dims, so a wave
  * works on 4 positions at once and the workgroup on 32; a batch of 4 such rounds (128
  * positions) has all its K and V rows requested before any is used.  Each of the 32 lane
