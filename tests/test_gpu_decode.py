@@ -124,6 +124,46 @@ def test_schedules_agree_and_match_oracle_over_steps():
         hip.close()
 
 
+@pytest.mark.parametrize("start", [381, 573])
+def test_steps_across_a_change_of_attention_schedule(start):
+    """Six teacher-forced steps over two layers that start three positions below a threshold of
+    the attention schedule (384: a head's positions go to 2 workgroups, 576: to 8): the rows
+    the kernel appended in the earlier steps are read by the later ones under the other
+    schedule, and by the workgroups that prefetch the next layer's rows into L2."""
+    steps, n_layers = 6, 2
+    layers = [S.Layer(5), S.Layer(6)]
+    norm = S.norm_weight(S.DIM, 98)
+    kv_max = start + steps + 2
+    k = np.zeros((26, kv_max, S.KV_DIM), np.float32)
+    v = np.zeros((26, kv_max, S.KV_DIM), np.float32)
+    for l in range(n_layers):
+        k[l, :start] = S.f32_normal((start, S.KV_DIM), 400 + l)
+        v[l, :start] = S.f32_normal((start, S.KV_DIM), 500 + l)
+    orc = cases.OracleBackend(threads=16)
+    orc.llm_open(layers, norm, kv_max, n_layers=n_layers)
+    for l in range(n_layers):
+        orc.kv_k[l], orc.kv_v[l] = k[l], v[l]
+    orc.pos = start
+    hip = H.Hip(kv_max=kv_max)
+    try:
+        hip.upload_decoder(layers, norm, n_layers)
+        hip.set_kv(k, v)
+        hip.lib.tts_hip_set_decode_mode(0)
+        hip.pos = start
+        e = S.f32_normal(S.DIM, 7)
+        for s_ in range(steps):
+            ref_h = orc.llm_forward(e)
+            got_h = hip.llm_forward(e)
+            assert_close(ref_h, got_h, f"step {s_} at position {start + s_}")
+            e = ref_h.copy()
+        gk, gv = hip.kv()
+        for l in range(n_layers):
+            assert_close(orc.kv_k[l, start:start + steps], gk[l, start:start + steps], f"k rows layer {l}")
+            assert_close(orc.kv_v[l, start:start + steps], gv[l, start:start + steps], f"v rows layer {l}")
+    finally:
+        hip.close()
+
+
 def test_26_layers_against_reference_fixture():
     """The committed fixture was written by the compiled reference: 26 layers
     cycling over two synthetic layers, 3 prefill rows then 2 decode steps
