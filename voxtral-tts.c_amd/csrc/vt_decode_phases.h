@@ -538,10 +538,16 @@ __device__ __forceinline__ void vt_kv_l2_prefetch(const vt_step_args &a, int lay
     const int total = 2 * a.pos * lines_per_row;                /* K and V rows 0 .. pos - 1 */
     const size_t base = (size_t)(a.first_layer + layer) * a.kv_max * VT_KV_DIM + (wg & 7) * VT_HEAD_DIM;
     unsigned acc = 0u;
-    for (int g = me; g < total; g += n_lanes) {
-        const int line = g % lines_per_row, row = (g / lines_per_row) % a.pos, kv = g / (lines_per_row * a.pos);
-        const float *p = (kv ? a.kv_v : a.kv_k) + base + (size_t)row * VT_KV_DIM + line * 32;
-        acc ^= *reinterpret_cast<const unsigned *>(p);
+    for (int g0 = me; g0 < total; g0 += 4 * n_lanes) {
+        unsigned v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int g = min(g0 + u * n_lanes, total - 1);     /* past the end: the last line once more */
+            const int line = g % lines_per_row, row = (g / lines_per_row) % a.pos, kv = g / (lines_per_row * a.pos);
+            const float *p = (kv ? a.kv_v : a.kv_k) + base + (size_t)row * VT_KV_DIM + line * 32;
+            v[u] = *reinterpret_cast<const unsigned *>(p);
+        }
+        acc ^= (v[0] ^ v[1]) ^ (v[2] ^ v[3]);
     }
     asm volatile("" ::"v"(acc));
 }
@@ -739,13 +745,23 @@ __device__ __forceinline__ void vt_w13_l2_prefetch(const vt_layer_dev &L, int bu
     const int per_wave = (per_wg + nw - 1) / nw;
     const int lines_per_row = VT_DIM * 2 / 128;
     const int total = per_x * nw * VT_L2_ROWS * lines_per_row;
+    /* four lines per turn, requested without a condition (a line that is not wanted is replaced by
+     * the first line of the matrix): with one conditional load per turn every turn waits for its
+     * own load */
     unsigned acc = 0u;
-    for (int g = me; g < total; g += n_lanes) {
-        const int line = g % lines_per_row, t = g / lines_per_row;
-        const int rr = t % VT_L2_ROWS, wv = (t / VT_L2_ROWS) % nw, i = t / (VT_L2_ROWS * nw);
-        const int row = ((wg & 7) + 8 * i) * per_wg + wv * per_wave + per_wave - VT_L2_ROWS + rr;
-        if (row < 2 * VT_FFN && !(rr == 0 && line < VT_L2_SKIP))
-            acc ^= *reinterpret_cast<const unsigned *>(L.w13 + (size_t)row * VT_DIM + line * 64);
+    for (int g0 = me; g0 < total; g0 += 4 * n_lanes) {
+        unsigned v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            const int g = g0 + u * n_lanes;
+            const int line = g % lines_per_row, t = g / lines_per_row;
+            const int rr = t % VT_L2_ROWS, wv = (t / VT_L2_ROWS) % nw, i = t / (VT_L2_ROWS * nw);
+            const int row = ((wg & 7) + 8 * i) * per_wg + wv * per_wave + per_wave - VT_L2_ROWS + rr;
+            const bool want = g < total && row < 2 * VT_FFN && !(rr == 0 && line < VT_L2_SKIP);
+            const size_t at = want ? (size_t)row * VT_DIM + line * 64 : 0;
+            v[u] = *reinterpret_cast<const unsigned *>(L.w13 + at);
+        }
+        acc ^= (v[0] ^ v[1]) ^ (v[2] ^ v[3]);
     }
     asm volatile("" ::"v"(acc));
 }
