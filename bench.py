@@ -626,8 +626,8 @@ def bench_layer(args):
         "config": {"workload": "one Mistral decoder layer, decode step at batch 1, KV cache of 512 positions ~N(0,1), "
                                "hidden ~N(0,1) (BASELINE.json configs[1])",
                    "weights": "bf16 N(0,0.02) seeded, truncated", "activations": "f32",
-                   "schedule": {0: "persistent whole-step kernel over one layer", 1: "one kernel per phase",
-                                2: "streaming kernel"}.get(args.mode, str(args.mode)),
+                   "schedule": {0: "persistent whole-step kernel over one layer",
+                                1: "one kernel per phase"}.get(args.mode, str(args.mode)),
                    "timed": "events on the library's stream, back-to-back launches, operands resident in HBM"},
         "hbm_gbps": round(gbps, 1),
         "roofline": {"kernel": "vt_decode_step_kernel (one layer)", "bound": "hbm", "achieved": round(gbps, 1),
@@ -682,7 +682,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", choices=("decode", "prefill", "acoustic", "frame", "codec", "matvec", "layer"), default="decode",
                     help="decode = the headline metric; prefill / acoustic = the other two configurations")
-    ap.add_argument("--mode", type=int, default=0, help="0 persistent kernel, 1 per-phase kernels, 2 streaming kernel")
+    ap.add_argument("--mode", type=int, default=0, choices=(0, 1), help="0 persistent kernel, 1 per-phase kernels")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one plain elementwise kernel (vt_add_kernel, a += b over 64 Mi floats: "
@@ -823,7 +823,7 @@ def main():
                         "hidden fed back through a 3072x3072 bf16 projection (BASELINE.json configs[2])",
             "layers": N_LAYERS, "prompt": PROMPT, "positions": [pos0, pos0 + K - 1],
             "weights": "bf16 N(0,0.02) seeded, truncated", "activations": "f32",
-            "schedule": ("persistent whole-step kernel", "one kernel per phase", "streaming whole-step kernel")[args.mode],
+            "schedule": ("persistent whole-step kernel", "one kernel per phase")[args.mode],
         },
         "frames_per_s": round(1000.0 / ms_step, 1),
         "hbm_gbps": round((bytes_launch + 2 * S.DIM * S.DIM) / (ms_step * 1e-3) / 1e9, 1),
@@ -831,7 +831,7 @@ def main():
         "ms_per_frame_normalised_6p8GB": round(ms_kernel * 6.8e9 / bytes_launch, 4),
         "ms_per_frame_host_pointers": round(ms_host, 4),
         "roofline": {
-            "kernel": ("vt_decode_step_kernel", "5 phase kernels per layer", "vt_decode_stream_kernel")[args.mode],
+            "kernel": ("vt_decode_step_kernel", "5 phase kernels per layer")[args.mode],
             "bound": "hbm",
             "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),

@@ -262,12 +262,22 @@ int tts_hip_load_safetensors(const char *path);
 int tts_hip_safetensors_probe(const char *path, const char *name, char *dtype8, int *rank,
                               long long *shape4, long long *nbytes);
 
-/* Decode schedule: 0 = persistent whole-step kernel (default), 1 = one kernel per
- * phase, 2 = streaming whole-step kernel (256-CU devices; experimental). */
+/* The table the loader uses when a checkpoint has no `time_embedding.inv_freq`: out[i] =
+ * expf(-logf(10000) * i / half_dim) for i < half_dim (the fallback of tts_acoustic_load,
+ * voxtral_tts_acoustic.c:48-60).  Host pointer; touches no GPU state. */
+void tts_hip_default_time_inv_freq(float *out, int half_dim);
+
+/* Decode schedule: 0 = persistent whole-step kernel (default; a device on which its grid cannot be
+ * resident at once runs schedule 1 instead), 1 = one kernel per phase.  Other values are an error
+ * and leave the schedule as it is. */
 void tts_hip_set_decode_mode(int mode);
-/* Spin budget of one grid barrier of the whole-step kernels, in ticks of the 100 MHz wall clock
- * (0 = the default of 0.2 s).  When it runs out every workgroup leaves the kernel, the call
- * reports an error and the result is invalid; the next call starts clean. */
+/* Spin budget of one grid barrier of the whole-step kernel, in ticks of the 100 MHz wall clock
+ * (0 = the default of 0.2 s).  When it runs out every workgroup leaves the kernel and the result is
+ * invalid.  Entry points with host pointers (tts_hip_llm_forward, tts_hip_generate_frame) report
+ * that themselves; after the asynchronous ones (tts_hip_llm_forward_device, tts_hip_layer_decode)
+ * it is reported, once, by the next call that waits for the stream: tts_hip_sync, tts_hip_to_host,
+ * tts_hip_to_device, tts_hip_memset, tts_hip_timer_stop_ms (which then returns a negative time).
+ * The report resets the barrier; the next step starts clean. */
 void tts_hip_set_barrier_timeout(unsigned long long ticks);
 /* Number of failed calls since init, and the text of the last failure. */
 int tts_hip_error_count(void);

@@ -59,23 +59,103 @@ void orc_embed_token_bf16(float *out, const uint16_t *emb, int token_id, int dim
 /* ---- linear (voxtral_tts_kernels.c:152-185 for one row of x,
  *              :187-211 + :127-138 for several) -----------------------------
  * Both reference paths start the accumulator at the bias (or 0) and add
- * w*x for k ascending; widening bf16 is exact, so one loop restates both. */
-void orc_linear_bf16(float *y, const float *x, const uint16_t *W_bf16,
-                     const float *bias, int seq_len, int in_dim, int out_dim) {
-    for (int s = 0; s < seq_len; s++) {
-        const float *xr = x + (size_t)s * in_dim;
-        float *yr = y + (size_t)s * out_dim;
+ * w*x for k ascending; widening bf16 is exact, so one loop restates both.
+ *
+ * Every output element is its own sequential chain (product rounded, then added, k
+ * ascending); the chains of different outputs are independent, so several of them are
+ * advanced side by side - eight output rows for a single row of x, and for several rows of x
+ * the rows of x as the lanes of a vector (x transposed into blocks of LANES columns) - which
+ * changes no bit of any result and takes the dependent-add latency off the critical path.
+ * tests/test_oracle_golden.py holds this against the compiled reference bit for bit. */
+typedef float v8f __attribute__((vector_size(32)));
+
+static void linear_one_row(float *y, const float *x, const uint16_t *W, const float *bias,
+                           int in_dim, int out_dim) {
 #pragma omp parallel for schedule(static) num_threads(g_threads) if (g_threads > 1)
-        for (int o = 0; o < out_dim; o++) {
-            const uint16_t *wr = W_bf16 + (size_t)o * in_dim;
-            float acc = bias ? bias[o] : 0.0f;
+    for (int o0 = 0; o0 < out_dim; o0 += 8) {
+        const int nb = out_dim - o0 < 8 ? out_dim - o0 : 8;
+        if (nb == 8) {
+            const uint16_t *w = W + (size_t)o0 * in_dim;
+            float a0 = bias ? bias[o0] : 0.0f, a1 = bias ? bias[o0 + 1] : 0.0f;
+            float a2 = bias ? bias[o0 + 2] : 0.0f, a3 = bias ? bias[o0 + 3] : 0.0f;
+            float a4 = bias ? bias[o0 + 4] : 0.0f, a5 = bias ? bias[o0 + 5] : 0.0f;
+            float a6 = bias ? bias[o0 + 6] : 0.0f, a7 = bias ? bias[o0 + 7] : 0.0f;
+            const size_t n = (size_t)in_dim;
             for (int k = 0; k < in_dim; k++) {
-                float p = widen(wr[k]) * xr[k];
-                acc = acc + p;
+                const float xv = x[k];
+                float p0 = widen(w[k]) * xv, p1 = widen(w[n + k]) * xv;
+                float p2 = widen(w[2 * n + k]) * xv, p3 = widen(w[3 * n + k]) * xv;
+                float p4 = widen(w[4 * n + k]) * xv, p5 = widen(w[5 * n + k]) * xv;
+                float p6 = widen(w[6 * n + k]) * xv, p7 = widen(w[7 * n + k]) * xv;
+                a0 = a0 + p0; a1 = a1 + p1; a2 = a2 + p2; a3 = a3 + p3;
+                a4 = a4 + p4; a5 = a5 + p5; a6 = a6 + p6; a7 = a7 + p7;
             }
-            yr[o] = acc;
+            y[o0] = a0; y[o0 + 1] = a1; y[o0 + 2] = a2; y[o0 + 3] = a3;
+            y[o0 + 4] = a4; y[o0 + 5] = a5; y[o0 + 6] = a6; y[o0 + 7] = a7;
+        } else {
+            for (int o = o0; o < o0 + nb; o++) {
+                const uint16_t *wr = W + (size_t)o * in_dim;
+                float acc = bias ? bias[o] : 0.0f;
+                for (int k = 0; k < in_dim; k++) {
+                    float p = widen(wr[k]) * x[k];
+                    acc = acc + p;
+                }
+                y[o] = acc;
+            }
         }
     }
+}
+
+/* rows s0 .. s0 + ns - 1 of x (ns <= 8 * NV) against every row of W; xt is x transposed,
+ * [in_dim][8 * NV] with zero padding */
+#define LINEAR_BLOCK(NV)                                                                        \
+static void linear_block_##NV(float *y, const v8f *xt, const uint16_t *W, const float *bias,    \
+                              int s0, int ns, int in_dim, int out_dim) {                        \
+    _Pragma("omp parallel for schedule(static) num_threads(g_threads) if (g_threads > 1)")      \
+    for (int o0 = 0; o0 < out_dim; o0 += 2) {                                                    \
+        const int two = o0 + 1 < out_dim;                                                        \
+        const uint16_t *w0 = W + (size_t)o0 * in_dim, *w1 = two ? w0 + in_dim : w0;             \
+        const float b0 = bias ? bias[o0] : 0.0f, b1 = bias ? bias[o0 + two] : 0.0f;             \
+        v8f a0[NV], a1[NV];                                                                      \
+        for (int v = 0; v < NV; v++)                                                             \
+            for (int l = 0; l < 8; l++) { a0[v][l] = b0; a1[v][l] = b1; }                        \
+        for (int k = 0; k < in_dim; k++) {                                                       \
+            const float f0 = widen(w0[k]), f1 = widen(w1[k]);                                    \
+            const v8f *xk = xt + (size_t)k * NV;                                                 \
+            for (int v = 0; v < NV; v++) {                                                       \
+                const v8f p0 = xk[v] * f0, p1 = xk[v] * f1;                                      \
+                a0[v] = a0[v] + p0;                                                              \
+                a1[v] = a1[v] + p1;                                                              \
+            }                                                                                    \
+        }                                                                                        \
+        for (int s = 0; s < ns; s++) {                                                           \
+            y[(size_t)(s0 + s) * out_dim + o0] = a0[s >> 3][s & 7];                              \
+            if (two) y[(size_t)(s0 + s) * out_dim + o0 + 1] = a1[s >> 3][s & 7];                 \
+        }                                                                                        \
+    }                                                                                            \
+}
+LINEAR_BLOCK(1)
+LINEAR_BLOCK(4)
+
+void orc_linear_bf16(float *y, const float *x, const uint16_t *W_bf16,
+                     const float *bias, int seq_len, int in_dim, int out_dim) {
+    if (seq_len == 1) {
+        linear_one_row(y, x, W_bf16, bias, in_dim, out_dim);
+        return;
+    }
+    const int nv = seq_len <= 8 ? 1 : 4, lanes = 8 * nv;
+    v8f *xt = aligned_alloc(32, sizeof(v8f) * (size_t)in_dim * nv);
+    if (!xt) abort();
+    for (int s0 = 0; s0 < seq_len; s0 += lanes) {
+        const int ns = seq_len - s0 < lanes ? seq_len - s0 : lanes;
+        float *t = (float *)xt;
+        for (int k = 0; k < in_dim; k++)
+            for (int l = 0; l < lanes; l++)
+                t[(size_t)k * lanes + l] = l < ns ? x[(size_t)(s0 + l) * in_dim + k] : 0.0f;
+        if (nv == 1) linear_block_1(y, xt, W_bf16, bias, s0, ns, in_dim, out_dim);
+        else linear_block_4(y, xt, W_bf16, bias, s0, ns, in_dim, out_dim);
+    }
+    free(xt);
 }
 
 /* ---- RMSNorm (voxtral_tts_kernels.c:333-349) ------------------------------ */

@@ -12,11 +12,16 @@
  * Pin status (what fixes each function besides this restatement):
  *   - all functions: bit-identical to the compiled reference sources
  *     (oracle/_ref, built from /root/reference by oracle/Makefile) in
- *     tests/test_oracle_vs_ref.py, and frozen in tests/golden/ fixtures
+ *     tests/test_oracle_golden.py, and frozen in tests/golden/ fixtures
  *     produced by that compiled reference.
  *   - the codec decoder functions (vt_oracle_codec.c): bit-identical to the compiled
  *     reference in tests/test_oracle_codec.py, frozen in tests/golden/codec.npz, and
  *     checked against closed forms and a float64 model of the whole decoder there.
+ *   - orc_default_time_inv_freq: the reference computes this table inside its checkpoint
+ *     loader (voxtral_tts_acoustic.c:48-60), which the compiled reference is never asked to
+ *     run; it is pinned by the mathematics instead (exact first entry, float64 closed form
+ *     within the fp32 argument's rounding, monotone, known middle and last entries) in
+ *     tests/test_oracle_math.py, and so is orc_time_embedding's cos|sin layout.
  *   - orc_linear_bf16 with seq_len > 1 follows the reference's no-BLAS
  *     triple loop (voxtral_tts_kernels.c:127-138).  The reference's BLAS
  *     build delegates the summation order to an unpinned third-party

@@ -303,6 +303,14 @@ def kernel_cases(b):
     bias = S.f32_normal(56, 1300, 0.1)
     out["linear3_bias"] = b.linear(x3, W, bias, 3)
     out["linear1_bias"] = b.linear(x3[:1].copy(), W, bias, 1)
+    # row counts that are no multiple of anything: 13 and 57 output rows, 5 / 19 / 40 rows of x
+    # (the oracle advances 8 output rows, or 8 / 32 rows of x, side by side)
+    W = S.bf16_normal((13, 200), 1400)
+    out["linear1_13rows"] = b.linear(S.f32_normal((1, 200), 1401), W, S.f32_normal(13, 1402, 0.1), 1)
+    W = S.bf16_normal((57, 328), 1410)
+    bias = S.f32_normal(57, 1411, 0.1)
+    for seq in (5, 19, 40):
+        out[f"linear{seq}_57rows"] = b.linear(S.f32_normal((seq, 328), 1420 + seq), W, bias if seq != 19 else None, seq)
     # rms norm
     x = S.f32_normal((3, S.DIM), 7)
     w = S.norm_weight(S.DIM, 8)

@@ -1,0 +1,173 @@
+"""The benchmark configurations at their full size against the oracle, through the C ABI:
+
+* 26 distinct layers, prefill of 512 random token ids on the GPU (tts_llm_prefill,
+  voxtral_tts_llm.c:277-392): K and V rows and the residual stream on a sample of rows;
+* 26 layers, 64-token prompt, 200 decode steps with each hidden fed back through a 3072 x 3072
+  bf16 projection (tts_llm_forward, voxtral_tts_llm.c:171-271): every step teacher-forced
+  against the oracle to the path's bound of 1e-3, then one free-running pass whose drift from the
+  oracle's chain is reported step by step;
+* 200 acoustic frames at seed 42 (tts_acoustic_forward, voxtral_tts_acoustic.c:268-373): exact
+  matches out of 7,400 codes, and for every differing code the float64 distance of the oracle's
+  latent from the FSQ rounding boundary.
+
+The oracle runs on 16 threads (bit-identical to one thread: output rows are independent)."""
+import ctypes as C
+import os
+from concurrent.futures import ThreadPoolExecutor
+
+import numpy as np
+import pytest
+
+import cases
+import hipsupport as H
+import vtsupport as S
+
+pytestmark = [pytest.mark.gpu, pytest.mark.timeout(900)]
+
+TOL = 1e-3              # max |d| / rms(ref) and ||d|| / ||ref|| per vector: the path's bound
+N_LAYERS = 26
+PROMPT = 64
+DECODE_STEPS = 200
+PREFILL_LEN = 512
+FRAMES = 200
+# A latent of the 7-step guided Euler flow differs from the oracle's by fp32 summation noise:
+# bound on max |x_gpu - x_oracle| over the 36 dims of a frame, and the same in the scaled units
+# of the FSQ rounding (x 10: 21 levels over [-1, 1]).
+LATENT_NOISE = 2e-5
+FSQ_NOISE = 10 * LATENT_NOISE
+
+
+def emb_row(token_id):
+    """Row `token_id` of the synthetic [131072, 3072] bf16 embedding table (as bench.py)."""
+    return S.bf16_to_f32(S.bf16_normal(S.DIM, 7_000_000 + int(token_id), 1.0))
+
+
+def close(ref, got, what, tol=TOL):
+    mx, l2 = S.rel_errors(ref, got)
+    assert np.all(np.isfinite(got)), what
+    assert mx < tol and l2 < tol, (what, mx, l2)
+    return mx, l2
+
+
+@pytest.fixture(scope="module")
+def backbone():
+    with ThreadPoolExecutor(16) as ex:
+        layers = list(ex.map(lambda i: S.Layer(1000 + i), range(N_LAYERS)))
+    norm = S.norm_weight(S.DIM, 99)
+    hip = H.Hip(kv_max=PREFILL_LEN + 8)
+    hip.upload_decoder(layers, norm, N_LAYERS)
+    orc = cases.OracleBackend(threads=16)
+    yield hip, orc, layers, norm
+    hip.close()
+
+
+def test_config3_prefill_512_tokens_26_layers(backbone):
+    hip, orc, layers, norm = backbone
+    ids = np.random.default_rng(11).integers(0, 131072, PREFILL_LEN)
+    with ThreadPoolExecutor(16) as ex:
+        embeds = np.stack(list(ex.map(emb_row, ids))).astype(np.float32)
+    orc.llm_open(layers, norm, PREFILL_LEN + 8, n_layers=N_LAYERS)
+    ref_x = orc.llm_prefill(embeds, want_x=True)
+    hip.pos = 0
+    got_x = hip.llm_prefill(embeds, want_x=True)
+    gk, gv = hip.kv()
+    worst = 0.0
+    rows = (0, 1, 2, 63, 64, 127, 128, 255, 300, 509, 510, 511)
+    for r in rows:
+        worst = max(worst, *close(ref_x[r], got_x[r], f"residual row {r}"))
+        for l in (0, 1, 12, 24, 25):
+            worst = max(worst, *close(orc.kv_k[l, r], gk[l, r], f"k layer {l} row {r}"))
+            worst = max(worst, *close(orc.kv_v[l, r], gv[l, r], f"v layer {l} row {r}"))
+    # every row of the last layer's cache, as one vector per row
+    for r in range(PREFILL_LEN):
+        worst = max(worst, *close(orc.kv_k[25, r], gk[25, r], f"k layer 25 row {r}"))
+    print(f"\nprefill 512 x 26 layers: worst of max|d|/rms and rel l2 over the sampled rows {worst:.3e}")
+
+
+def test_config2_decode_200_steps_teacher_forced_and_free_running(backbone):
+    hip, orc, layers, norm = backbone
+    lib = hip.lib
+    proj = S.bf16_normal((S.DIM, S.DIM), 31337)
+    ids = np.random.default_rng(7).integers(0, 131072, PROMPT)
+    prompt = np.stack([emb_row(t) for t in ids]).astype(np.float32)
+    orc.llm_open(layers, norm, PREFILL_LEN + 8, n_layers=N_LAYERS)
+    orc.llm_prefill(prompt)
+    hip.pos = 0
+    hip.llm_prefill(prompt)                     # rows 0..63 of the cache; later rows are stale and never read
+
+    e0 = S.f32_normal(S.DIM, 4242)
+    # teacher-forced: both sides get the oracle chain's input at every step
+    e = e0.copy()
+    ref_h, worst = [], (0.0, 0.0)
+    for s in range(DECODE_STEPS):
+        r = orc.llm_forward(e)
+        g = hip.llm_forward(e)
+        mx, l2 = close(r, g, f"teacher-forced step {s} (position {PROMPT + s})")
+        worst = (max(worst[0], mx), max(worst[1], l2))
+        ref_h.append(r)
+        e = orc.linear(r.reshape(1, -1), proj, None, 1)[0]
+    gk, gv = hip.kv()
+    for l in (0, 12, 25):
+        for r in (PROMPT, PROMPT + 99, PROMPT + DECODE_STEPS - 1):
+            close(orc.kv_k[l, r], gk[l, r], f"appended k row {r} layer {l}")
+            close(orc.kv_v[l, r], gv[l, r], f"appended v row {r} layer {l}")
+    print(f"\ndecode, 200 teacher-forced steps: max|d|/rms {worst[0]:.3e}, rel l2 {worst[1]:.3e}")
+
+    # free-running: the GPU feeds its own hidden back through the projection on the device
+    d_proj = H.DevBuf.from_numpy(lib, proj)
+    d_e = H.DevBuf.from_numpy(lib, e0)
+    d_h = H.DevBuf(lib, S.DIM * 4)
+    drift = []
+    for s in range(DECODE_STEPS):
+        lib.tts_hip_llm_forward_device(d_h.ptr, d_e.ptr, PROMPT + s)
+        lib.tts_hip_linear_bf16(d_e.ptr, d_h.ptr, None, 1, S.DIM, S.DIM, d_proj.ptr)
+        drift.append(S.rel_errors(ref_h[s], d_h.to_numpy(np.float32, S.DIM)))
+    hip.check()
+    drift = np.array(drift)
+    assert np.all(np.isfinite(drift))
+    assert drift[0, 0] < TOL and drift[0, 1] < TOL            # step 0 has the same input on both sides
+    report = ", ".join(f"step {s}: {drift[s, 0]:.2e}" for s in (0, 1, 5, 10, 25, 50, 100, 150, 199))
+    print(f"decode, free-running drift (max|d|/rms against the oracle's own chain): {report}; "
+          f"largest {drift[:, 0].max():.2e} at step {int(drift[:, 0].argmax())}")
+    for b in (d_proj, d_e, d_h):
+        b.free()
+
+
+def test_config4_acoustic_200_frames_codes(backbone):
+    """Runs after the backbone tests in the same session (one global context)."""
+    hip = backbone[0]
+    ac = S.Acoustic(50)
+    hip.upload_acoustic(ac)
+    orc = cases.OracleBackend(threads=16)
+    orc.ac_open(ac)
+    st = C.c_uint64(0)
+    S.oracle().orc_rng_seed(C.byref(st), 42)
+    equal = total = n_end = 0
+    worst_latent, margins = 0.0, []
+    for f in range(FRAMES):
+        h = S.f32_normal(S.DIM, 20 + f)
+        rc, rst, rx = orc.acoustic_forward(h, seed=42 if f == 0 else None, want_x=True)
+        if rc[0] == 1:                                  # END_AUDIO: the reference draws no noise
+            x0 = np.zeros(S.ACOUSTIC_DIM, np.float32)
+            n_end += 1
+        else:
+            x0 = np.zeros(S.ACOUSTIC_DIM, np.float32)
+            S.oracle().orc_randn_fill(C.byref(st), S.fp(x0), S.ACOUSTIC_DIM)
+        assert int(st.value) == int(rst), f"frame {f}: the host RNG left the oracle's sequence"
+        codes, x = hip.acoustic_frame(h, x0)
+        assert codes[0] == rc[0], (f, codes[0], rc[0])
+        total += S.CODES
+        equal += int(np.sum(codes == rc))
+        if rc[0] != 1:
+            worst_latent = max(worst_latent, float(np.max(np.abs(x.astype(np.float64) - rx))))
+        for i in np.nonzero(codes[1:] != rc[1:])[0]:
+            scaled = (np.clip(np.float64(rx[i]), -1.0, 1.0) + 1.0) / 2.0 * 20.0 + 0.5
+            m = abs(scaled - round(scaled))
+            margins.append((f, int(i), int(codes[1 + i]), int(rc[1 + i]), m))
+            assert abs(int(codes[1 + i]) - int(rc[1 + i])) == 1, margins[-1]
+            assert m < FSQ_NOISE, margins[-1]
+    print(f"\nacoustic, {FRAMES} frames at seed 42: {equal} of {total} codes equal, {n_end} END frames, "
+          f"max |latent - oracle| {worst_latent:.2e}; differing codes (frame, dim, gpu, oracle, margin): {margins}")
+    assert total == FRAMES * S.CODES
+    assert worst_latent < LATENT_NOISE, worst_latent
+    assert equal >= total - 8            # a handful of latents on a boundary at most

@@ -167,3 +167,40 @@ def test_audio_embed_sum_uses_cumulative_offsets():
     out = B.audio_embed(S.f32_to_bf16_trunc(emb), codes)
     assert np.array_equal(out[:S.CODES], np.ones(S.CODES, np.float32))
     assert not np.any(out[S.CODES:])
+
+
+def _check_time_inv_freq(f):
+    """What the mathematics fixes for f[i] = exp(-log(10000) i / 1536) evaluated in fp32
+    (voxtral_tts_acoustic.c:48-60): f[0] is exactly 1; the fp32 argument (-logf(1e4) * i) / 1536
+    carries at most three roundings (logf, product, quotient: 3 * 2^-24 relative, |argument| <= 9.21,
+    so 1.65e-6 absolute), expf adds an ulp: every entry lies within 2e-6 relative of the float64
+    value.  An index off by one is 6e-3 away, a dropped sign or a wrong base much more."""
+    half = S.DIM // 2
+    assert f.shape == (half,) and f.dtype == np.float32
+    assert f[0] == np.float32(1.0)
+    ref = np.exp(-np.log(10000.0) * np.arange(half, dtype=np.float64) / half)
+    assert np.max(np.abs(f.astype(np.float64) / ref - 1.0)) < 2e-6
+    assert np.all(np.diff(f) < 0)
+    assert abs(float(f[half - 1]) - 1.0060e-4) < 1e-8
+    assert abs(float(f[half // 2]) - 1e-2) < 1e-7          # the middle entry is 10000^-0.5
+
+
+def test_default_time_inv_freq_closed_form():
+    f = np.zeros(S.DIM // 2, np.float32)
+    S.oracle().orc_default_time_inv_freq(S.fp(f), S.DIM // 2)
+    _check_time_inv_freq(f)
+
+
+def test_time_embedding_is_cos_then_sin_of_t_times_freq():
+    """out[i] = cos(t f_i), out[1536 + i] = sin(t f_i) (voxtral_tts_acoustic.c:166-176), against
+    float64 on a table pinned above; t = 0 gives (1, 0)."""
+    f = np.zeros(S.DIM // 2, np.float32)
+    S.oracle().orc_default_time_inv_freq(S.fp(f), S.DIM // 2)
+    out = np.zeros(S.DIM, np.float32)
+    S.oracle().orc_time_embedding(S.fp(f), np.float32(0.0), S.fp(out), S.DIM)
+    assert np.array_equal(out[:S.DIM // 2], np.ones(S.DIM // 2, np.float32)) and not np.any(out[S.DIM // 2:])
+    t = np.float32(3) / np.float32(7)
+    S.oracle().orc_time_embedding(S.fp(f), t, S.fp(out), S.DIM)
+    ang = (t * f).astype(np.float64)
+    assert np.max(np.abs(out[:S.DIM // 2] - np.cos(ang))) < 1e-6
+    assert np.max(np.abs(out[S.DIM // 2:] - np.sin(ang))) < 1e-6

@@ -12,6 +12,7 @@ import torch
 from safetensors.torch import save_file
 
 import hipsupport as H
+import vtsupport as S
 
 
 def probe(lib, path, name):
@@ -134,3 +135,12 @@ def test_load_needs_an_initialised_backend(lib, tmp_path):
     if not H.load_package().ctx().initialized:
         assert lib.tts_hip_load_safetensors(str(p).encode()) == -1
         assert lib.tts_hip_error_count() == n0 + 1
+
+
+def test_fallback_time_frequencies_follow_the_closed_form(lib):
+    """The table the loader computes when a checkpoint lacks `time_embedding.inv_freq`
+    (voxtral_tts_acoustic.c:48-60), checked against the mathematics, not against the oracle."""
+    from test_oracle_math import _check_time_inv_freq
+    f = np.zeros(S.DIM // 2, np.float32)
+    lib.tts_hip_default_time_inv_freq(f.ctypes.data, S.DIM // 2)
+    _check_time_inv_freq(f)

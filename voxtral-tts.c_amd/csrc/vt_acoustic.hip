@@ -823,6 +823,7 @@ static int enqueue_frame(ac_work *w, const float *d_or_h_hidden, const float *x0
 
 static void finish_frame(const ac_work *w, int *out_codes, float *out_x) {
     VT_TRYV(hipStreamSynchronize(g_vt.stream));
+    if (vt_step_poll_abort()) return;      /* the backbone step in front of this frame was abandoned */
     VT_TRYV(hipMemcpy(out_codes, w->codes, sizeof(int) * (1 + VT_AC_DIM_IN), hipMemcpyDeviceToHost));
     if (out_x) VT_TRYV(hipMemcpy(out_x, w->x, sizeof(float) * VT_AC_DIM_IN, hipMemcpyDeviceToHost));
     if (out_codes[0] == 1) {                            /* END_AUDIO */

@@ -91,14 +91,10 @@ static int init_context(int kv_cache_max) {
     g_vt.n_cu = prop.multiProcessorCount;
     g_vt.grid = g_vt.n_cu / VT_KV_HEADS * VT_KV_HEADS;
     if (g_vt.grid < VT_KV_HEADS) { vt_set_error("device has too few compute units"); return -1; }
-    /* more than half of a CU's LDS per workgroup => exactly one workgroup per CU */
-    size_t lds_cu = prop.maxSharedMemoryPerMultiProcessor, lds_wg = prop.sharedMemPerBlock;
-    size_t want = lds_cu / 2 + 4096;
-    g_vt.step_dyn_lds = (want + 24 * 1024 <= lds_wg) ? want : 0;
     if (getenv("TTS_HIP_VERBOSE"))
         fprintf(stderr, "  HIP: %s, %d CUs, %.1f GB, LDS %zu/%zu KB, grid %d\n", prop.gcnArchName,
-                g_vt.n_cu, (double)prop.totalGlobalMem / (1 << 30), lds_wg >> 10, lds_cu >> 10,
-                g_vt.grid);
+                g_vt.n_cu, (double)prop.totalGlobalMem / (1 << 30), (size_t)prop.sharedMemPerBlock >> 10,
+                (size_t)prop.maxSharedMemoryPerMultiProcessor >> 10, g_vt.grid);
 
     VT_TRY(hipStreamCreateWithFlags(&g_vt.stream, hipStreamNonBlocking));
     VT_TRY(hipEventCreate(&g_vt.ev0));
@@ -350,16 +346,19 @@ extern "C" int tts_hip_upload_acoustic_weights(void *acoustic_ptr) {
 
 extern "C" void tts_hip_to_device(void *d_dst, const void *h_src, size_t bytes) {
     (void)hipStreamSynchronize(g_vt.stream);
+    (void)vt_step_poll_abort();
     (void)vt_check(hipMemcpy(d_dst, h_src, bytes, hipMemcpyHostToDevice), "tts_hip_to_device");
 }
 
 extern "C" void tts_hip_to_host(void *h_dst, const void *d_src, size_t bytes) {
     (void)hipStreamSynchronize(g_vt.stream);
+    (void)vt_step_poll_abort();
     (void)vt_check(hipMemcpy(h_dst, d_src, bytes, hipMemcpyDeviceToHost), "tts_hip_to_host");
 }
 
 extern "C" void tts_hip_memset(void *d_ptr, int value, size_t bytes) {
     (void)hipStreamSynchronize(g_vt.stream);
+    (void)vt_step_poll_abort();
     (void)vt_check(hipMemset(d_ptr, value, bytes), "tts_hip_memset");
 }
 
@@ -370,10 +369,14 @@ extern "C" void tts_hip_free_ptr(void *d_ptr) {
 }
 
 extern "C" void tts_hip_sync(void) {
-    (void)vt_check(hipDeviceSynchronize(), "tts_hip_sync");
+    if (vt_check(hipDeviceSynchronize(), "tts_hip_sync")) return;
+    (void)vt_step_poll_abort();
 }
 
-extern "C" void tts_hip_set_decode_mode(int mode) { g_vt.decode_mode = mode; }
+extern "C" void tts_hip_set_decode_mode(int mode) {
+    if (mode != 0 && mode != 1) { vt_set_error("tts_hip_set_decode_mode: unknown schedule %d", mode); return; }
+    g_vt.decode_mode = mode;
+}
 extern "C" void tts_hip_set_barrier_timeout(unsigned long long ticks) { g_vt.bar_timeout = ticks; }
 extern "C" int tts_hip_error_count(void) { return g_vt.error_count; }
 extern "C" const char *tts_hip_last_error(void) { return g_vt.last_error; }
@@ -387,5 +390,6 @@ extern "C" float tts_hip_timer_stop_ms(void) {
     if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "timer stop")) return ms;
     if (vt_check(hipEventSynchronize(g_vt.ev1), "timer sync")) return ms;
     (void)vt_check(hipEventElapsedTime(&ms, g_vt.ev0, g_vt.ev1), "timer elapsed");
+    if (vt_step_poll_abort()) return -1.f;      /* a step of the timed region was abandoned: no figure */
     return ms;
 }

@@ -9,15 +9,18 @@
  *           requested between arriving at a barrier and waiting on it, so the
  *           HBM stream does not stop while the tiny activation vectors are
  *           exchanged between workgroups.
- *   mode 1  one kernel per phase (5 launches per layer), same numerics.
- *   mode 2  the streaming kernel of vt_decode_stream.hip (256-CU devices only):
- *           weight streaming decoupled from synchronisation, 6 stream waves + 1
- *           control wave per CU.  Correct and reproducible, but not yet faster
- *           than mode 0 (its control path pays the CU's shared memory queue on
- *           every hand-over); opt-in.
+ *   mode 1  one kernel per phase (5 launches per layer), same numerics; also the
+ *           schedule a device falls to when the whole grid of mode 0 cannot be
+ *           resident at once.
+ *
+ * A barrier of mode 0 that runs out of its spin budget raises a flag on the device
+ * and every workgroup leaves the kernel.  The host learns of it at its next
+ * synchronising call (vt_step_poll_abort): the failed step is counted as an error,
+ * the flag and the barrier epochs are reset, and the next launch starts clean.
  */
 #include "vt_state.h"
 
+#include <stdlib.h>
 #include <string.h>
 
 /* ---- persistent whole-step kernel -------------------------------------------- */
@@ -206,24 +209,19 @@ int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
 
     const dim3 grid(g_vt.grid), block(VT_STEP_THREADS);
     hipStream_t st = g_vt.stream;
-    if (g_vt.decode_mode == 2) {
-        if (!vt_stream_supported()) { vt_set_error("decode step: the streaming schedule needs a 256-CU device"); return -1; }
-        return vt_run_step_stream(a);
-    } else if (g_vt.decode_mode == 0) {
+    if (g_vt.decode_mode != 0 && g_vt.decode_mode != 1) {
+        vt_set_error("decode step: unknown schedule %d (0 = whole-step kernel, 1 = one kernel per phase)",
+                     g_vt.decode_mode);
+        return -1;
+    }
+    if (g_vt.decode_mode == 0 && vt_step_resident()) {
         vt_grid_sync gs;
         gs.flags = g_vt.d_bar_flags;
         gs.abort_flag = g_vt.d_abort;
         gs.epoch = g_vt.bar_epoch + 1u;
         gs.timeout = g_vt.bar_timeout ? g_vt.bar_timeout : 20000000ull;   /* default 0.2 s of the 100 MHz wall clock */
         g_vt.bar_epoch += 5u * (unsigned)n_layers;
-        static int attr_set = 0;
-        if (!attr_set && g_vt.step_dyn_lds) {
-            if (vt_check(hipFuncSetAttribute((const void *)vt_decode_step_kernel,
-                                             hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             (int)g_vt.step_dyn_lds), "hipFuncSetAttribute"))
-                g_vt.step_dyn_lds = 0;
-            attr_set = 1;
-        }
+        g_vt.step_pending = 1;
         hipLaunchKernelGGL(vt_decode_step_kernel, grid, block, g_vt.step_dyn_lds, st, a, gs);
     } else {
         if (vt_check(hipMemsetAsync(g_vt.d_att_cnt, 0, sizeof(unsigned) * n_layers * VT_KV_HEADS, st),
@@ -242,7 +240,55 @@ int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
     return vt_check(hipGetLastError(), "decode step launch");
 }
 
-/* Reads the abort flag of the persistent kernel after a synchronisation. */
+/* Whether every workgroup of the whole-step kernel can be resident at once, which its grid
+ * barrier needs: asked of the runtime once per context, for the kernel as built (registers, static
+ * LDS) with the dynamic LDS it is launched with.  The dynamic LDS is sized from the kernel's real
+ * static LDS so that static + dynamic exceeds half a CU's LDS, i.e. so that a CU never takes a
+ * second workgroup of this kernel whatever its register count; where a workgroup may not ask for
+ * that much the pin is left out (the registers of 8 waves of this kernel fill more than half a
+ * CU's file, which has the same effect).  Not resident: the step runs as one kernel per phase. */
+int vt_step_resident(void) {
+    if (g_vt.step_checked) return g_vt.step_fits;
+    g_vt.step_checked = 1;
+    g_vt.step_fits = 0;
+    hipFuncAttributes fa;
+    if (vt_check(hipFuncGetAttributes(&fa, (const void *)vt_decode_step_kernel), "hipFuncGetAttributes")) return 0;
+    hipDeviceProp_t prop;
+    if (vt_check(hipGetDeviceProperties(&prop, g_vt.device), "hipGetDeviceProperties")) return 0;
+    const size_t lds_cu = prop.maxSharedMemoryPerMultiProcessor;
+    size_t dyn = 0;
+    if (fa.sharedSizeBytes <= lds_cu / 2) {
+        dyn = lds_cu / 2 + 1024 - fa.sharedSizeBytes;
+        dyn = (dyn + 1023) / 1024 * 1024;
+        if (fa.sharedSizeBytes + dyn > (size_t)prop.sharedMemPerBlockOptin && fa.sharedSizeBytes + dyn > prop.sharedMemPerBlock) dyn = 0;
+        if (dyn && hipFuncSetAttribute((const void *)vt_decode_step_kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn) != hipSuccess) {
+            (void)hipGetLastError();
+            dyn = 0;
+        }
+    }
+    int per_cu = 0;
+    if (vt_check(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, vt_decode_step_kernel, VT_STEP_THREADS, dyn),
+                 "hipOccupancyMaxActiveBlocksPerMultiprocessor")) return 0;
+    if (per_cu < 1 && dyn) {            /* the pin itself does not fit: without it */
+        dyn = 0;
+        if (vt_check(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, vt_decode_step_kernel, VT_STEP_THREADS, dyn),
+                     "hipOccupancyMaxActiveBlocksPerMultiprocessor")) return 0;
+    }
+    g_vt.step_dyn_lds = dyn;
+    g_vt.step_fits = (long long)per_cu * g_vt.n_cu >= g_vt.grid;
+    if (getenv("TTS_HIP_VERBOSE"))
+        fprintf(stderr, "  HIP: whole-step kernel: %d VGPRs, %zu B static + %zu B dynamic LDS, %d workgroup(s) per CU, grid %d %s\n",
+                fa.numRegs, (size_t)fa.sharedSizeBytes, dyn, per_cu, g_vt.grid,
+                g_vt.step_fits ? "resident" : "NOT resident: one kernel per phase instead");
+    if (!g_vt.step_fits)
+        fprintf(stderr, "tts_hip: the whole-step decode kernel cannot be resident on this device "
+                        "(%d workgroups per CU x %d CUs < grid %d): running one kernel per phase\n",
+                per_cu, g_vt.n_cu, g_vt.grid);
+    return g_vt.step_fits;
+}
+
+/* After a timed-out barrier: count the failure, clear the flag and the epochs. */
 static int step_aborted(int flag) {
     if (!flag) return 0;
     vt_set_error("decode step: grid barrier timed out; kernel left early, result invalid");
@@ -251,6 +297,17 @@ static int step_aborted(int flag) {
     (void)hipStreamSynchronize(g_vt.stream);
     g_vt.bar_epoch = 0;
     return -1;
+}
+
+/* Called by every entry point right after it has synchronised with the library's stream: if a
+ * whole-step kernel ran since the last look, reads its abort flag (a 4-byte copy) and reports a
+ * timed-out barrier like any other failed call.  Returns -1 if a step had been abandoned. */
+int vt_step_poll_abort(void) {
+    if (!g_vt.initialized || !g_vt.step_pending) return 0;
+    g_vt.step_pending = 0;
+    int flag = 0;
+    if (vt_check(hipMemcpy(&flag, g_vt.d_abort, sizeof flag, hipMemcpyDeviceToHost), "abort flag read")) return -1;
+    return step_aborted(flag);
 }
 
 #ifdef VT_TRACE
@@ -280,6 +337,7 @@ extern "C" void tts_hip_llm_forward(float *out_hidden, const float *input_embed,
     VT_TRYV(hipStreamSynchronize(st));
     int flag;
     memcpy(&flag, pin_out + VT_DIM, sizeof flag);
+    g_vt.step_pending = 0;
     if (step_aborted(flag)) return;
     memcpy(out_hidden, pin_out, sizeof(float) * VT_DIM);
 }

@@ -260,6 +260,14 @@ static float *st_f32(const st_file *f, const char *name, long long elems) {
 
 /* Looks one tensor up (no GPU involved): 0 and its dtype / rank / shape / byte size, 1 when the
  * file has no such tensor, -1 when the file cannot be read. */
+/* The time-embedding frequencies a checkpoint without `time_embedding.inv_freq` gets:
+ * f[i] = exp(-log(10000) i / half_dim) in fp32, operations in the order of
+ * voxtral_tts_acoustic.c:48-60.  Host only. */
+extern "C" void tts_hip_default_time_inv_freq(float *out, int half_dim) {
+    const float theta = 10000.0f;
+    for (int i = 0; i < half_dim; i++) out[i] = expf(-logf(theta) * (float)i / (float)half_dim);
+}
+
 extern "C" int tts_hip_safetensors_probe(const char *path, const char *name, char *dtype8, int *rank,
                                          long long *shape4, long long *nbytes) {
     st_file f;
@@ -431,7 +439,7 @@ extern "C" int tts_hip_load_safetensors(const char *path) {
                 /* not in the checkpoint: the closed form of voxtral_tts_acoustic.c:48-60 */
                 float *tf = (float *)malloc(sizeof(float) * (VT_DIM / 2));
                 ok = tf != NULL;
-                for (int i = 0; ok && i < VT_DIM / 2; i++) tf[i] = expf(-logf(10000.0f) * (float)i / (float)(VT_DIM / 2));
+                if (ok) tts_hip_default_time_inv_freq(tf, VT_DIM / 2);
                 ac->time_inv_freq = tofree[nfree - 1] = tf;
             }
             ac->input_proj_bf16 = (uint16_t *)st_bf16(&f, "acoustic_transformer.input_projection.weight", (long long)VT_DIM * VT_AC_DIM_IN);

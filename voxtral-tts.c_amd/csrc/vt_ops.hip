@@ -193,8 +193,11 @@ void vt_launch_linear(float *d_y, const float *d_x, const uint16_t *d_W, const f
 
 /* Rows of activations against an aligned weight matrix go to the matrix cores:
  * (hi, lo) planes of x, K cut into enough ranges to fill the device, partial
- * planes summed in a fixed order.  Returns 0 when the shape does not qualify. */
-static int linear_mfma(float *d_y, const float *d_x, const uint16_t *d_W, int seq_len, int in_dim, int out_dim) {
+ * planes summed in a fixed order.  linear_mfma_plan says whether the shape qualifies, into how
+ * many ranges K is cut and how many bytes of work area (partial planes, then the two activation
+ * planes) the launches need; linear_mfma_run queues them on that work area. */
+static int linear_mfma_plan(const float *d_y, const float *d_x, const uint16_t *d_W, int seq_len, int in_dim,
+                            int out_dim, int *splits_out, size_t *bytes_out) {
     if (seq_len < 8 || !vt_gemm_shape_ok(seq_len, out_dim, in_dim, 1) ||
         (((uintptr_t)d_W | (uintptr_t)d_x | (uintptr_t)d_y) & 15))
         return 0;
@@ -205,13 +208,30 @@ static int linear_mfma(float *d_y, const float *d_x, const uint16_t *d_W, int se
         if (vt_gemm_shape_ok(seq_len, out_dim, in_dim, cand[i])) splits = cand[i];
     const size_t n_in = (size_t)seq_len * in_dim, n_out = (size_t)seq_len * out_dim;
     const size_t part_bytes = splits > 1 ? sizeof(float) * n_out * splits : 0;
-    unsigned char *base = (unsigned char *)vt_scratch(part_bytes + 2 * sizeof(uint16_t) * n_in);
-    if (!base) return -1;
+    *splits_out = splits;
+    *bytes_out = part_bytes + 2 * sizeof(uint16_t) * n_in;
+    return 1;
+}
+
+static void linear_mfma_run(unsigned char *base, float *d_y, const float *d_x, const uint16_t *d_W, int seq_len,
+                            int in_dim, int out_dim, int splits) {
+    const size_t n_in = (size_t)seq_len * in_dim, n_out = (size_t)seq_len * out_dim;
+    const size_t part_bytes = splits > 1 ? sizeof(float) * n_out * splits : 0;
     float *part = splits > 1 ? (float *)base : d_y;
     uint16_t *hi = (uint16_t *)(base + part_bytes), *lo = hi + n_in;
     vt_launch_split(hi, lo, d_x, n_in);
     vt_launch_gemm(part, hi, lo, d_W, seq_len, out_dim, in_dim, splits);
     if (splits > 1) vt_launch_sum_planes(d_y, part, splits, n_out, n_out);
+}
+
+/* Returns 0 when the shape does not qualify, 1 when queued, -1 on error. */
+static int linear_mfma(float *d_y, const float *d_x, const uint16_t *d_W, int seq_len, int in_dim, int out_dim) {
+    int splits;
+    size_t bytes;
+    if (!linear_mfma_plan(d_y, d_x, d_W, seq_len, in_dim, out_dim, &splits, &bytes)) return 0;
+    unsigned char *base = (unsigned char *)vt_scratch(bytes);
+    if (!base) return -1;
+    linear_mfma_run(base, d_y, d_x, d_W, seq_len, in_dim, out_dim, splits);
     return 1;
 }
 
@@ -474,7 +494,7 @@ extern "C" void tts_hip_causal_attention_prefill(float *d_out, const float *d_Q,
     if (start_pos < 0) { vt_set_error("tts_hip_causal_attention_prefill: negative start_pos"); return; }
     if (n_heads == VT_HEADS && n_kv_heads == VT_KV_HEADS && head_dim == VT_HEAD_DIM && seq_len >= 8 &&
         !(((uintptr_t)d_out | (uintptr_t)d_Q | (uintptr_t)d_K | (uintptr_t)d_V) & 15)) {
-        vt_launch_prefill_attention(d_out, NULL, NULL, d_Q, VT_Q_DIM, d_K, d_V, seq_len, start_pos);
+        vt_launch_prefill_attention(d_out, NULL, NULL, d_Q, VT_Q_DIM, d_K, d_V, seq_len, start_pos, scale);
         return;
     }
     vt_launch_attention(d_out, d_Q, d_K, d_V, seq_len, start_pos, start_pos + seq_len, 1, n_heads,

@@ -264,8 +264,8 @@ static size_t pa_lds_bytes(void) {
 
 /* Q rows are q_stride floats apart; out / (out_hi, out_lo) are [S,4096], each optional. */
 void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
-                                 int q_stride, const float *d_K, const float *d_V, int S, int start_pos) {
-    const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
+                                 int q_stride, const float *d_K, const float *d_V, int S, int start_pos,
+                                 float scale) {
     static int attr_set = 0;
     if (!attr_set) {
         if (vt_check(hipFuncSetAttribute((const void *)vt_prefill_attention_kernel<PA_NSPLIT, PA_HPW>,
@@ -317,7 +317,7 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
         hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(ew_blocks(S * VT_QKV_DIM / 4)), dim3(256), 0, st,
                            wide, sp_qkv, S * VT_QKV_DIM, q, kc, vc, g_vt.d_rope, start_pos, seq_len);
-        vt_launch_prefill_attention(NULL, hi, lo, q, VT_Q_DIM, kc, vc, seq_len, start_pos);
+        vt_launch_prefill_attention(NULL, hi, lo, q, VT_Q_DIM, kc, vc, seq_len, start_pos, VT_ATT_SCALE);
         vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
         vt_launch_residual_norm_split(x, part, sp_wo, ps, L->ffn_norm, hi, lo, seq_len);
         if (tail_cols) {
@@ -384,7 +384,7 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
             vt_launch_gemm_ex(out + (size_t)S * 2 * VT_FFN, tail, (size_t)S * tail, hi, lo,
                               W[2] + (size_t)main_cols * VT_DIM, S, tail, VT_DIM, 4);
         } else if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], SP[which]);
-        else vt_launch_prefill_attention(out, NULL, NULL, q, VT_Q_DIM, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu, S, 0);
+        else vt_launch_prefill_attention(out, NULL, NULL, q, VT_Q_DIM, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu, S, 0, VT_ATT_SCALE);
     }
     if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;
     if (vt_check(hipEventSynchronize(g_vt.ev1), "bench sync")) return -1.f;

@@ -7,6 +7,7 @@
 #define VT_STATE_H
 
 #include <hip/hip_runtime.h>
+#include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
 
@@ -40,6 +41,8 @@ struct vt_state {
     int n_cu;
     int grid;                     /* workgroups of the persistent kernels */
     size_t step_dyn_lds;          /* dynamic LDS that pins one workgroup per CU */
+    int step_checked, step_fits;  /* residency of the whole-step kernel's grid, asked once per context */
+    int step_pending;             /* a whole-step kernel was launched and its abort flag not yet looked at */
     hipStream_t stream;
     hipEvent_t ev0, ev1;
     int decode_mode;
@@ -96,11 +99,14 @@ void vt_launch_attention(float *d_out, const float *d_Q, const float *d_K, const
                          int n_kv_heads, int head_dim, float scale, int kv_stride, int q_stride);
 void vt_launch_add(float *d_a, const float *d_b, int n);
 void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
-                                 int q_stride, const float *d_K, const float *d_V, int S, int start_pos);
+                                 int q_stride, const float *d_K, const float *d_V, int S, int start_pos,
+                                 float scale);
+/* the model's attention scale, 1/sqrt(head_dim), computed like the CPU path does (voxtral_tts_llm.c:189) */
+#define VT_ATT_SCALE (1.0f / sqrtf((float)VT_HEAD_DIM))
 void vt_codec_free(void);
 float vt_bench_codec(int which, int iters);
-int vt_stream_supported(void);
-int vt_run_step_stream(const vt_step_args &a);
+int vt_step_resident(void);
+int vt_step_poll_abort(void);
 int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
                 const float *d_final_norm, const float *d_in, float *d_out, int pos);
 
