@@ -80,7 +80,9 @@ def test_audio_embed_bit_exact(session):
         assert np.array_equal(got, orc.audio_embed(table, codes))
 
 
-FSQ_NOISE = 2e-4        # scaled units (21 levels over [-1, 1]): 10 x the latent's fp32 noise bound of 2e-5
+# scaled units of the FSQ rounding (21 levels over [-1, 1]): 10 x the bound of 1e-4 on the latent's
+# accumulated fp32 noise that tests/test_gpu_fullsize.py holds over 200 frames (measured 5.9e-5)
+FSQ_NOISE = 1e-3
 
 
 def fsq_margin(x):
