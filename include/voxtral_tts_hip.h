@@ -262,6 +262,17 @@ int tts_hip_load_safetensors(const char *path);
 int tts_hip_safetensors_probe(const char *path, const char *name, char *dtype8, int *rank,
                               long long *shape4, long long *nbytes);
 
+/* y[seq_len, out_dim] = x[seq_len, in_dim] W[out_dim, in_dim]^T on device pointers, like
+ * tts_hip_linear_bf16 with device buffers and the same kernels, for callers that cannot allocate
+ * device memory (code under HIP graph capture, tight serving loops, harnesses that forbid it).  No
+ * counterpart in the reference.  The work area of the matrix-core path (two bf16 planes of x and
+ * the partial planes of a K cut) is a fixed array of 16 MiB that every GPU the library runs on
+ * holds until the process ends; a product that needs more is refused with an error (use
+ * tts_hip_linear_bf16).  Calls no hipMalloc / hipFree.  All calls on one GPU share the array:
+ * calls that overlap on one GPU race.  Asynchronous on the library's stream; 0 / -1. */
+int tts_hip_linear_bf16_noalloc(float *d_y, const float *d_x, int seq_len, int in_dim, int out_dim,
+                                const void *d_W);
+
 /* The table the loader uses when a checkpoint has no `time_embedding.inv_freq`: out[i] =
  * expf(-logf(10000) * i / half_dim) for i < half_dim (the fallback of tts_acoustic_load,
  * voxtral_tts_acoustic.c:48-60).  Host pointer; touches no GPU state. */

@@ -126,6 +126,7 @@ SIGNATURES = {
     "tts_hip_codec_decode": (None, [vp, C.c_int, C.POINTER(f32p), i32p]),
     "tts_hip_codec_decode_device": (C.c_int, [vp, C.c_int, vp]),
     "tts_hip_load_safetensors": (C.c_int, [C.c_char_p]),
+    "tts_hip_linear_bf16_noalloc": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, vp]),
     "tts_hip_default_time_inv_freq": (None, [vp, C.c_int]),
     "tts_hip_safetensors_probe": (C.c_int, [C.c_char_p, C.c_char_p, C.c_char_p, C.c_void_p,
                                             C.c_void_p, C.c_void_p]),

@@ -235,6 +235,61 @@ static int linear_mfma(float *d_y, const float *d_x, const uint16_t *d_W, int se
     return 1;
 }
 
+/* ---- the same product for callers that cannot allocate ----------------------------------
+ * The work area of the matrix-core path lives in a fixed array in device memory instead of the
+ * context's growing buffer, so this entry point reaches no hipMalloc / hipFree (nor any routine
+ * that allocates) on any path.  Every device that loads the library holds its own copy of the
+ * array at its own address for the life of the process; the address is looked up once per device,
+ * with that device current, and only that pointer is ever handed to kernels.  The array keeps the
+ * last call's contents; nothing in it has to start at zero (the activation planes and every
+ * element of every partial plane that is read are written by the call itself).  Calls that overlap
+ * on one device would share the array: the library has one stream and is not thread-safe. */
+#define VT_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
+#define VT_STATIC_MAX_DEVICES 16
+static __device__ __align__(256) unsigned char vt_static_scratch[VT_STATIC_SCRATCH_BYTES];
+static unsigned char *s_static_ptr[VT_STATIC_MAX_DEVICES];
+
+static unsigned char *static_scratch(void) {
+    int dev = -1;
+    if (vt_check(hipGetDevice(&dev), "hipGetDevice")) return NULL;
+    if (dev < 0 || dev >= VT_STATIC_MAX_DEVICES) {
+        vt_set_error("tts_hip_linear_bf16_noalloc: device %d beyond the %d this build keeps an address for", dev,
+                     VT_STATIC_MAX_DEVICES);
+        return NULL;
+    }
+    if (!s_static_ptr[dev]) {
+        void *p = NULL;
+        if (vt_check(hipGetSymbolAddress(&p, HIP_SYMBOL(vt_static_scratch)), "hipGetSymbolAddress")) return NULL;
+        s_static_ptr[dev] = (unsigned char *)p;
+    }
+    return s_static_ptr[dev];
+}
+
+extern "C" int tts_hip_linear_bf16_noalloc(float *d_y, const float *d_x, int seq_len, int in_dim, int out_dim,
+                                           const void *d_W) {
+    if (!g_vt.initialized) { vt_set_error("tts_hip_linear_bf16_noalloc: backend not initialised"); return -1; }
+    if (!d_y || !d_x || !d_W || seq_len < 1 || in_dim < 1 || out_dim < 1) {
+        vt_set_error("tts_hip_linear_bf16_noalloc: bad arguments");
+        return -1;
+    }
+    int splits;
+    size_t bytes;
+    if (!linear_mfma_plan(d_y, d_x, (const uint16_t *)d_W, seq_len, in_dim, out_dim, &splits, &bytes)) {
+        /* few rows or an unaligned shape: the row kernels, which use no work area at all */
+        vt_launch_linear(d_y, d_x, (const uint16_t *)d_W, NULL, seq_len, in_dim, out_dim);
+        return vt_check(hipGetLastError(), "tts_hip_linear_bf16_noalloc") ? -1 : 0;
+    }
+    if (bytes > VT_STATIC_SCRATCH_BYTES) {
+        vt_set_error("tts_hip_linear_bf16_noalloc: %d x %d x %d needs %zu bytes of work area, the fixed one has %zu; "
+                     "use tts_hip_linear_bf16", seq_len, out_dim, in_dim, bytes, (size_t)VT_STATIC_SCRATCH_BYTES);
+        return -1;
+    }
+    unsigned char *base = static_scratch();
+    if (!base) return -1;
+    linear_mfma_run(base, d_y, d_x, (const uint16_t *)d_W, seq_len, in_dim, out_dim, splits);
+    return vt_check(hipGetLastError(), "tts_hip_linear_bf16_noalloc") ? -1 : 0;
+}
+
 extern "C" int tts_hip_split_planes(uint16_t *d_hi, uint16_t *d_lo, const float *d_x, size_t n) {
     if (!g_vt.initialized) { vt_set_error("tts_hip_split_planes: backend not initialised"); return -1; }
     if (!d_hi || !d_lo || !d_x || (n & 1) || (((uintptr_t)d_x) & 7) || (((uintptr_t)d_hi | (uintptr_t)d_lo) & 3)) {
