@@ -59,6 +59,77 @@ def measured_traffic(workload):
         return None
 
 
+TRAFFIC_SOURCE = "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command, scaled by a copy kernel; not measured by this run)"
+
+
+def find_cblas():
+    """A CBLAS sgemm found at run time, as (callable, description, threads), or (None, reason, 0).
+    Looks for a system OpenBLAS, the OpenBLAS that scipy bundles (exported with a scipy_ prefix) and
+    MKL, in that order; nothing is installed or built for it."""
+    import ctypes.util
+    import glob
+    tries = []
+    for name in ("openblas", "mkl_rt"):
+        path = ctypes.util.find_library(name)
+        if path:
+            tries.append((path, "cblas_sgemm", "openblas_get_config", "openblas_get_num_threads"))
+    try:
+        import scipy
+        libs = os.path.join(os.path.dirname(os.path.dirname(scipy.__file__)), "scipy.libs")
+        for path in sorted(glob.glob(os.path.join(libs, "libscipy_openblas*.so*"))):
+            tries.append((path, "scipy_cblas_sgemm", "scipy_openblas_get_config", "scipy_openblas_get_num_threads"))
+    except ImportError:
+        pass
+    for path, sym, cfg, nthr in tries:
+        try:
+            lib = C.CDLL(path)
+            fn = getattr(lib, sym)
+        except (OSError, AttributeError):
+            continue
+        fn.restype = None
+        fn.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_int,
+                       C.c_void_p, C.c_int, C.c_float, C.c_void_p, C.c_int]
+        desc, threads = os.path.basename(path), 0
+        try:
+            g = getattr(lib, cfg)
+            g.restype = C.c_char_p
+            desc += ": " + g().decode()
+            t = getattr(lib, nthr)
+            t.restype = C.c_int
+            threads = int(t())
+        except AttributeError:
+            pass
+        return fn, desc, threads
+    return None, "no CBLAS library found (libopenblas, scipy's bundled OpenBLAS, libmkl_rt)", 0
+
+
+def cpu_blas_linears(sgemm, shapes, weights, m, budget_s):
+    """The reference's seq_len > 1 linear in its BLAS build (voxtral_tts_kernels.c:187-198 and
+    112-140): widen the whole bf16 matrix to fp32 (tts_bf16_to_f32_buf, :49-53), then
+    cblas_sgemm(RowMajor, NoTrans, Trans, seq, out, in, 1, x, in, W, in, 0, y, out).  Times that pair
+    for every (out, in) of `shapes` once (twice if the budget allows) on m rows of N(0,1) activations;
+    returns the seconds per shape."""
+    orc = S.oracle()
+    orc.orc_bf16_to_f32_buf.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+    out = {}
+    t_start = time.time()
+    for (name, n, k), W in zip(shapes, weights):
+        x = S.f32_normal((m, k), 77 + k)
+        y = np.zeros((m, n), np.float32)
+        wf = np.empty((n, k), np.float32)
+        best = None
+        for rep in range(2):
+            t0 = time.time()
+            orc.orc_bf16_to_f32_buf(wf.ctypes.data, W.ctypes.data, n * k)
+            sgemm(101, 111, 112, m, n, k, 1.0, x.ctypes.data, k, wf.ctypes.data, k, 0.0, y.ctypes.data, n)
+            dt = time.time() - t0
+            best = dt if best is None else min(best, dt)
+            if time.time() - t_start > budget_s:
+                break
+        out[name] = best
+    return out
+
+
 def emb_row(token_id):
     """Row `token_id` of the synthetic [131072, 3072] bf16 embedding table."""
     return S.bf16_to_f32(S.bf16_normal(S.DIM, 7_000_000 + int(token_id), 1.0))
@@ -125,6 +196,39 @@ def prefill_flops(seq):
     return gemm, attn
 
 
+REF_LINEARS = (("wq", S.Q_DIM, S.DIM), ("wk", S.KV_DIM, S.DIM), ("wv", S.KV_DIM, S.DIM), ("wo", S.DIM, S.Q_DIM),
+               ("w1", S.FFN, S.DIM), ("w3", S.FFN, S.DIM), ("w2", S.DIM, S.FFN))
+
+
+def prefill_cpu_baseline(layers, budget_s, m=PREFILL_LEN, calls=N_LAYERS):
+    """The seq_len > 1 products of the reference's BLAS build on this host: the seven linears of one
+    layer at m rows (widen + sgemm each), times `calls` layer passes.  Attention, norms and RoPE
+    (under 2 % of the reference's prefill) are left out and the figure says so."""
+    sgemm, desc, threads = find_cblas()
+    if sgemm is None:
+        return {"value": None, "unit": "ms", "cores": 0, "kind": "reference-noblas", "sample": desc}
+    # layer after layer (distinct weights, so nothing is served from a cache) until the budget is used
+    t0, per, n_done = time.time(), {}, 0
+    for l in layers:
+        one = cpu_blas_linears(sgemm, REF_LINEARS, [getattr(l, n) for n, _, _ in REF_LINEARS], m, budget_s)
+        for k, v in one.items():
+            per[k] = per.get(k, 0.0) + v
+        n_done += 1
+        if time.time() - t0 > 0.7 * budget_s:
+            break
+    per = {k: v / n_done for k, v in per.items()}
+    layer_s = sum(per.values())
+    return {
+        "value": round(layer_s * calls * 1e3, 1), "unit": "ms", "cores": threads or (os.cpu_count() or 1),
+        "kind": "port", "library": desc,
+        "sample": f"the seven linears of one layer at {m} rows as the reference's BLAS build runs them "
+                  f"(tts_bf16_to_f32_buf of the whole matrix + cblas_sgemm, voxtral_tts_kernels.c:187-198, 112-140): "
+                  f"{layer_s * 1e3:.0f} ms per layer (mean over {n_done} layers), x {calls}; attention / norms / RoPE "
+                  f"not included",
+        "per_linear_ms": {k: round(v * 1e3, 1) for k, v in per.items()},
+    }
+
+
 def bench_prefill(args):
     """BASELINE.json config "Backbone prefill": 26 layers, 512 random token ids, causal GQA
     attention.  A step is one whole prefill into an empty cache; inputs are resident in HBM."""
@@ -181,7 +285,7 @@ def bench_prefill(args):
             "bound": "mfma",
             "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": measured_traffic("prefill"),
+            "traffic": measured_traffic("prefill"), "traffic_source": TRAFFIC_SOURCE,
             "flops_per_layer": 2 * PREFILL_LEN * LAYER_WEIGHT_ELEMS,
             "ms_per_layer": round(ms_gemm_layer, 4),
             "executed_over_algorithmic": 2.0,
@@ -191,9 +295,10 @@ def bench_prefill(args):
         "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
         "cpu_baseline": None,
     }
+    if args.cpu_seconds > 0:
+        out["cpu_baseline"] = prefill_cpu_baseline(layers, args.cpu_seconds)
     if args.cpu_seconds > 0 and S.have_ref():
-        # the reference's own tts_llm_prefill (triple-loop linear, no BLAS in this build), single thread,
-        # on the first n_cpu tokens of the same prompt; the cost per token is flat in this range
+        # parity of the GPU prefill against the reference's own tts_llm_prefill on the first tokens
         n_cpu = 2
         b = cases.RefBackend()
         b.llm_open(layers, final_norm, 16)
@@ -206,14 +311,15 @@ def bench_prefill(args):
         gk, gv = hip.kv()
         errs = [S.rel_errors(rk[l, r], gk[l, r]) for l in (0, N_LAYERS - 1) for r in range(n_cpu)]
         errs += [S.rel_errors(rv[l, r], gv[l, r]) for l in (0, N_LAYERS - 1) for r in range(n_cpu)]
-        out["cpu_baseline"] = {
-            "value": round(dt / n_cpu * PREFILL_LEN * 1e3, 1), "unit": "ms/prefill", "cores": 1, "kind": "reference",
+        out["cpu_reference_noblas"] = {
+            "value": round(dt / n_cpu * PREFILL_LEN * 1e3, 1), "unit": "ms/prefill", "cores": 1, "kind": "reference-noblas",
             "sample": f"tts_llm_prefill of the first {n_cpu} tokens through all 26 layers ({dt:.1f} s), scaled "
-                      f"linearly to 512 tokens; no-BLAS build of the reference",
+                      f"linearly to 512 tokens; no-BLAS build of the reference (its BLAS build needs <cblas.h>)",
         }
         out["parity"] = {"max_abs_over_rms": float(f"{max(e[0] for e in errs):.3e}"),
                          "rel_l2": float(f"{max(e[1] for e in errs):.3e}"),
-                         "checked": f"K and V rows 0..{n_cpu - 1} of layers 0 and 25", "against": "reference"}
+                         "checked": f"K and V rows 0..{n_cpu - 1} of layers 0 and 25", "against": "reference",
+                         "full_size": "tests/test_gpu_fullsize.py holds all 512 rows x 26 layers to 1e-3 against the CPU port"}
         assert out["parity"]["max_abs_over_rms"] < 1e-3, out["parity"]
     hip.close()
     print(json.dumps(out))
@@ -293,7 +399,7 @@ def bench_acoustic(args):
             "bound": "hbm",
             "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": measured_traffic("acoustic"),
+            "traffic": measured_traffic("acoustic"), "traffic_source": TRAFFIC_SOURCE,
             "bytes_per_layer": AC_LAYER_BYTES, "ms_per_layer": round(ms_layer, 4),
             "per_phase_alone": per_phase,
             "note": "ms_per_layer: the four launches in order, rotating over the 3 layers; per_phase_alone: one "
@@ -303,8 +409,39 @@ def bench_acoustic(args):
         "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
         "cpu_baseline": None,
     }
+    if args.cpu_seconds > 0:
+        # 14 velocity evaluations per frame (7 Euler steps x 2 guidance branches), each 3 layers at 3 rows
+        base = prefill_cpu_baseline(ac.layers, args.cpu_seconds, m=3, calls=14 * 3)
+        base["unit"] = "ms/frame"
+        out["cpu_baseline"] = base
+    if args.cpu_seconds > 0:
+        # parity: as many frames as fit the budget against the CPU port on all host threads (bit-identical
+        # to one thread), noise from the restated host RNG at seed 42
+        orc = cases.OracleBackend(threads=min(16, os.cpu_count() or 1))
+        orc.ac_open(ac)
+        st2 = C.c_uint64(0)
+        S.oracle().orc_rng_seed(C.byref(st2), 42)
+        equal = total = 0
+        worst = 0.0
+        t0 = time.time()
+        f = 0
+        while f < 200 and time.time() - t0 < args.cpu_seconds:
+            h = S.f32_normal(S.DIM, 20 + f)
+            rc, _, rx = orc.acoustic_forward(h, seed=42 if f == 0 else None, want_x=True)
+            x0 = np.zeros(S.ACOUSTIC_DIM, np.float32)
+            if rc[0] != 1:
+                S.oracle().orc_randn_fill(C.byref(st2), S.fp(x0), S.ACOUSTIC_DIM)
+            g, gx = hip.acoustic_frame(h, x0)
+            equal += int(np.sum(g == rc))
+            total += S.CODES
+            if rc[0] != 1:
+                worst = max(worst, float(np.max(np.abs(gx.astype(np.float64) - rx))))
+            f += 1
+        out["parity"] = {"codes_equal": equal, "codes": total, "frames": f, "max_latent_diff": float(f"{worst:.3e}"),
+                         "against": "port", "full_size": "tests/test_gpu_fullsize.py runs all 200 frames (7,400 codes)"}
+        assert worst < 1e-4, worst
     if args.cpu_seconds > 0 and S.have_ref():
-        # one frame of the reference's tts_acoustic_forward (14 velocity evaluations), single thread
+        # one frame of the reference's tts_acoustic_forward (14 velocity evaluations), single thread, no BLAS
         b = cases.RefBackend()
         b.ac_open(ac)
         t0 = time.time()
@@ -313,9 +450,8 @@ def bench_acoustic(args):
         b.ac_close()
         g = np.zeros(S.CODES, np.int32)
         lib.tts_hip_acoustic_frame(g.ctypes.data, d_h[0].ptr, d_x[0].ptr, None)
-        out["cpu_baseline"] = {"value": round(dt * 1e3, 1), "unit": "ms/frame", "cores": 1, "kind": "reference",
-                               "sample": "one frame of tts_acoustic_forward at seed 42 (same hidden state and noise)"}
-        out["parity"] = {"codes_equal": int(np.sum(g == rc)), "codes": int(S.CODES), "against": "reference"}
+        out["cpu_reference_noblas"] = {"value": round(dt * 1e3, 1), "unit": "ms/frame", "cores": 1, "kind": "reference-noblas",
+                                       "sample": "one frame of tts_acoustic_forward at seed 42 (same hidden state and noise)"}
         assert np.array_equal(g, rc), (g, rc)
     hip.close()
     print(json.dumps(out))
@@ -398,7 +534,7 @@ def bench_codec(args):
             "bound": "mfma",
             "achieved": round(achieved, 1), "peak": MFMA_F32_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_F32_PEAK_TFLOPS, 4),
-            "traffic": measured_traffic("codec"),
+            "traffic": measured_traffic("codec"), "traffic_source": TRAFFIC_SOURCE,
             "flops_per_layer": layer_fl, "ms_per_layer": round(layer_ms, 4), "per_shape": per_shape,
         },
         "flops_per_utterance": fl,
@@ -563,7 +699,7 @@ def bench_matvec(args):
                    "timed": "events on the library's stream, operands resident in HBM"},
         "per_shape": per_shape,
         "roofline": {"kernel": "vt_matvec_kernel (131072x3072)", "bound": "hbm", "achieved": big["gbps"],
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": big["frac"], "traffic": measured_traffic("matvec"),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": big["frac"], "traffic": measured_traffic("matvec"), "traffic_source": TRAFFIC_SOURCE,
                      "bytes_per_launch": big["bytes"], "ms_per_launch": round(big["us"] / 1e3, 5)},
         "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
         "cpu_baseline": None,
@@ -675,6 +811,87 @@ def bench_layer(args):
     print(json.dumps(out))
 
 
+def other_workloads(hip, kv_max):
+    """Short runs of the other BASELINE.json configurations inside the default line, so that one
+    command shows every kernel's rate: the three single products (configs[0]), one decoder layer at
+    512 cached positions (configs[1]), the 512-token prefill (configs[3]) and the acoustic frame
+    (configs[4]).  Weights of the single products are a constant fill (timing only; their parity is
+    in tests/); the backbone runs use the 26 uploaded layers, each launch on the next layer so that
+    weights come from HBM.  The full lines, with CPU baseline and parity, are --workload <name>."""
+    lib = hip.lib
+    w = {}
+    # configs[0]
+    for n, k, what in MATVEC_SHAPES:
+        copies = 8 if 2 * n * k < (512 << 20) else 1
+        d_W = H.DevBuf(lib, copies * 2 * n * k)
+        lib.tts_hip_memset(d_W.ptr, 0x3c, copies * 2 * n * k)          # bf16 0x3c3c = 0.0115
+        d_x = H.DevBuf.from_numpy(lib, S.f32_normal((1, k), 42))
+        d_y = H.DevBuf(lib, 4 * n)
+        ms = lib.tts_hip_bench_matvec(d_y.ptr, d_x.ptr, d_W.ptr, n * k, copies, k, n, 24)
+        nbytes = 2 * n * k + 4 * k + 4 * n
+        w[f"matvec {n}x{k}"] = {"config": 0, "kernel": "vt_matvec_kernel", "us": round(ms * 1e3, 2), "launches": 24,
+                                "achieved": round(nbytes / ms / 1e6, 1), "unit": "GB/s",
+                                "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+        for b in (d_W, d_x, d_y):
+            b.free()
+    # configs[1]: one layer per launch at position 512, walking through the 26 layers
+    pos = PREFILL_LEN
+    d_x = H.DevBuf.from_numpy(lib, S.f32_normal(S.DIM, 42))
+    for l in range(N_LAYERS):
+        lib.tts_hip_layer_decode(l, d_x.ptr, pos)
+    lib.tts_hip_sync()
+    lib.tts_hip_timer_start()
+    n_l = 2 * N_LAYERS
+    for i in range(n_l):
+        lib.tts_hip_layer_decode(i % N_LAYERS, d_x.ptr, pos)
+    ms = lib.tts_hip_timer_stop_ms() / n_l
+    nbytes = LAYER_WEIGHT_BYTES + 2 * S.DIM * 4 + 2 * (pos + 1) * S.KV_DIM * 4 + 2 * S.KV_DIM * 4 + 2 * S.DIM * 4
+    w["layer decode, 512 cached positions"] = {
+        "config": 1, "kernel": "vt_decode_step_kernel (one layer per launch)", "us": round(ms * 1e3, 2), "launches": n_l,
+        "achieved": round(nbytes / ms / 1e6, 1), "unit": "GB/s", "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    d_x.free()
+    # configs[3]: whole prefills, then the product kernel per projection shape
+    d_e = H.DevBuf.from_numpy(lib, S.f32_normal((PREFILL_LEN, S.DIM), 11))
+    lib.tts_hip_llm_prefill(d_e.ptr, PREFILL_LEN, 0)
+    lib.tts_hip_sync()
+    lib.tts_hip_timer_start()
+    for _ in range(3):
+        lib.tts_hip_llm_prefill(d_e.ptr, PREFILL_LEN, 0)
+    ms = lib.tts_hip_timer_stop_ms() / 3
+    gemm_fl, attn_fl = prefill_flops(PREFILL_LEN)
+    ms_layer = sum(lib.tts_hip_bench_kernel(i, 26) for i in range(4))
+    achieved = 2.0 * PREFILL_LEN * LAYER_WEIGHT_ELEMS / ms_layer / 1e9
+    w["prefill, 512 tokens x 26 layers"] = {
+        "config": 3, "kernel": "vt_gemm_mfma_kernel (the projection launches of one layer)", "ms": round(ms, 3), "launches": 3,
+        "tokens_per_s": round(PREFILL_LEN / (ms * 1e-3), 1), "tflops_whole_prefill": round((gemm_fl + attn_fl) / ms / 1e9, 1),
+        "us_products_per_layer": round(ms_layer * 1e3, 1), "achieved": round(achieved, 1), "unit": "TFLOP/s",
+        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "attention_us_per_layer": round(lib.tts_hip_bench_kernel(4, 26) * 1e3, 1)}
+    d_e.free()
+    # configs[4]
+    ac = S.Acoustic(50)
+    hip.upload_acoustic(ac)
+    st = C.c_uint64(0)
+    S.oracle().orc_rng_seed(C.byref(st), 42)
+    x0 = np.zeros(S.ACOUSTIC_DIM, np.float32)
+    S.oracle().orc_randn_fill(C.byref(st), S.fp(x0), S.ACOUSTIC_DIM)
+    d_h, d_x0 = H.DevBuf.from_numpy(lib, S.f32_normal(S.DIM, 20)), H.DevBuf.from_numpy(lib, x0)
+    codes = np.zeros(S.CODES, np.int32)
+    for _ in range(2):
+        lib.tts_hip_acoustic_frame(codes.ctypes.data, d_h.ptr, d_x0.ptr, None)
+    t0 = time.perf_counter()
+    for _ in range(10):
+        lib.tts_hip_acoustic_frame(codes.ctypes.data, d_h.ptr, d_x0.ptr, None)
+    ms = (time.perf_counter() - t0) * 1e3 / 10
+    ms_layer = lib.tts_hip_bench_kernel(14, 30)
+    achieved = AC_LAYER_BYTES / ms_layer / 1e6
+    w["acoustic frame"] = {
+        "config": 4, "kernel": "vt_ac_phase_kernel (the launches of one layer, in order)", "ms": round(ms, 4), "launches": 10,
+        "frame_gbps": round(acoustic_frame_bytes() / ms / 1e6, 1), "us_per_layer": round(ms_layer * 1e3, 1),
+        "achieved": round(achieved, 1), "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4)}
+    hip.check()
+    return w
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -684,6 +901,8 @@ def main():
                     help="decode = the headline metric; prefill / acoustic = the other two configurations")
     ap.add_argument("--mode", type=int, default=0, choices=(0, 1), help="0 persistent kernel, 1 per-phase kernels")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--no-workloads", action="store_true",
+                    help="leave the short runs of the other configurations out of the default line")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch one plain elementwise kernel (vt_add_kernel, a += b over 64 Mi floats: "
                          "512 MiB read, 256 MiB written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
@@ -718,7 +937,7 @@ def main():
     t_gen = time.time() - t0
 
     n_cpu = 6 if args.cpu_seconds > 0 else 0
-    kv_max = PROMPT + n_cpu + 2 * (W + K) + 8
+    kv_max = max(PROMPT + n_cpu + 2 * (W + K) + 8, PREFILL_LEN + 8)     # room for the 512-row workloads below
     hip = H.Hip(kv_max=kv_max)
     lib = hip.lib
     lib.tts_hip_set_decode_mode(args.mode)
@@ -836,11 +1055,14 @@ def main():
             "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
+            "traffic_source": TRAFFIC_SOURCE if args.traffic_kib is None else "--traffic-kib",
             "bytes_per_launch": int(bytes_launch),
             "ms_per_launch": round(ms_kernel, 4),
         },
         "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
     }
+    if not args.no_workloads:
+        out["workloads"] = other_workloads(hip, kv_max)
     if n_cpu:
         base, parity = cpu_baseline(layers, final_norm, kv_k, kv_v, kv_max, rec_e, rec_h, args.cpu_seconds)
         out["cpu_baseline"] = base

@@ -98,6 +98,32 @@ def test_causal_attention_tiles(hip, orc, seq, start):
         b.free()
 
 
+def test_causal_attention_honours_the_callers_scale(hip):
+    """The reference's entry takes the softmax scale as an argument (voxtral_tts_cuda.h:142-146);
+    the matrix-core path (8 or more queries, aligned pointers) must use it like the generic path,
+    not the model's 1/sqrt(128)."""
+    seq, scale = 40, 0.03
+    Q = S.f32_normal((seq, S.Q_DIM), 811)
+    K = S.f32_normal((seq, S.KV_DIM), 812)
+    V = S.f32_normal((seq, S.KV_DIM), 813)
+    ref = np.zeros_like(Q)
+    S.oracle().orc_causal_attention(S.fp(ref), S.fp(Q), S.fp(K), S.fp(V), seq, seq, S.HEADS, S.KV_HEADS,
+                                    S.HEAD_DIM, scale, 0, 0)
+    dQ, dK, dV = (H.DevBuf.from_numpy(hip.lib, a) for a in (Q, K, V))
+    dO = H.DevBuf(hip.lib, Q.nbytes)
+    hip.lib.tts_hip_causal_attention_prefill(dO.ptr, dQ.ptr, dK.ptr, dV.ptr, seq, 0, S.HEADS,
+                                             S.KV_HEADS, S.HEAD_DIM, scale)
+    hip.lib.tts_hip_sync()
+    hip.check()
+    got = dO.to_numpy(np.float32, Q.shape)
+    rows_close(ref, got, "attention with scale 0.03", tight=1e-4)
+    # and the two scales really give different answers on this input
+    ref_default = cases.OracleBackend(threads=16).causal_attention(Q, K, V, seq, seq, 0)
+    assert np.max(np.abs(ref_default - ref)) > 1e-2
+    for b in (dQ, dK, dV, dO):
+        b.free()
+
+
 def test_attention_first_key_only_and_equal_keys(hip):
     """Closed forms: query 0 sees one key, so its output is V row 0 of its KV head;
     with all keys equal every query returns the mean of the visible V rows."""
