@@ -9,6 +9,7 @@
  * into one [18432, 3072] matrix so that a (gate, up) pair is adjacent.
  */
 #include "vt_state.h"
+#include "vt_gemm.h"
 
 #include <math.h>
 #include <stdlib.h>
@@ -149,6 +150,30 @@ extern "C" int tts_hip_init(int kv_cache_max) {
     return 0;
 }
 
+static void free_frag(vt_layer_frag *g) {
+    (void)hipFree(g->wqkv); (void)hipFree(g->wo); (void)hipFree(g->w13); (void)hipFree(g->w2);
+    memset(g, 0, sizeof *g);
+}
+
+/* The fragment-order copies of a complete backbone layer (6.05 GB for 26 layers, next to the 6.05 GB of
+ * the row-major ones).  A failure leaves the layer without them: the prefill then multiplies from the
+ * row-major matrices with the 128 x 128 tile kernel. */
+static int build_frag(vt_layer_frag *g, const vt_layer_dev *l) {
+    free_frag(g);
+    struct { uint16_t **dst; const uint16_t *src; int n, k; } m[4] = {
+        {&g->wqkv, l->wqkv, VT_QKV_DIM, VT_DIM}, {&g->wo, l->wo, VT_DIM, VT_Q_DIM},
+        {&g->w13, l->w13, 2 * VT_FFN, VT_DIM}, {&g->w2, l->w2, VT_DIM, VT_FFN}};
+    for (int i = 0; i < 4; i++) {
+        if (!(*m[i].dst = (uint16_t *)vt_dev_alloc((size_t)m[i].n * m[i].k * 2))) { free_frag(g); return -1; }
+        vt_launch_frag_layout(*m[i].dst, m[i].src, m[i].n, m[i].k);
+    }
+    if (vt_check(hipGetLastError(), "fragment layout launch") || vt_check(hipStreamSynchronize(g_vt.stream), "fragment layout")) {
+        free_frag(g);
+        return -1;
+    }
+    return 0;
+}
+
 static void free_layer(vt_layer_dev *l) {
     (void)hipFree((void *)l->wqkv); (void)hipFree((void *)l->wo);
     (void)hipFree((void *)l->w13); (void)hipFree((void *)l->w2);
@@ -160,7 +185,7 @@ static void free_layer(vt_layer_dev *l) {
 static void teardown(void) {
     (void)hipDeviceSynchronize();
     vt_codec_free();
-    for (int i = 0; i < TTS_HIP_DEC_LAYERS; i++) free_layer(&g_vt.h_layers[i]);
+    for (int i = 0; i < TTS_HIP_DEC_LAYERS; i++) { free_layer(&g_vt.h_layers[i]); free_frag(&g_vt.h_frag[i]); }
     for (int i = 0; i < TTS_HIP_AC_LAYERS; i++) free_layer(&g_vt.ac.layers[i]);
     void *ptrs[] = {g_vt.d_layers, g_vt.d_dec_norm, g_vt.d_tok_emb, g_vt.ac.input_proj,
                     g_vt.ac.time_proj, g_vt.ac.llm_proj, g_vt.ac.semantic_out,
@@ -262,7 +287,8 @@ extern "C" int tts_hip_upload_llm_layer(int layer, const tts_hip_host_layer_t *s
     }
     (void)hipStreamSynchronize(g_vt.stream);
     const int bad = upload_layer(&g_vt.h_layers[layer], src);
-    if (bad) free_layer(&g_vt.h_layers[layer]);          /* incomplete: the backbone ends in front of it */
+    if (bad) { free_layer(&g_vt.h_layers[layer]); free_frag(&g_vt.h_frag[layer]); }   /* incomplete: the backbone ends in front of it */
+    else (void)build_frag(&g_vt.h_frag[layer], &g_vt.h_layers[layer]);
     if (publish_dec_layers()) return -1;
     return bad ? -1 : 0;
 }
@@ -294,10 +320,12 @@ extern "C" int tts_hip_upload_llm_weights_n(void *decoder_ptr, int n_layers) {
         if (i < n_layers && upload_layer(&g_vt.h_layers[i], &dec->layers[i])) {
             fprintf(stderr, "tts_hip: failed to upload LLM layer %d\n", i);
             free_layer(&g_vt.h_layers[i]);
+            free_frag(&g_vt.h_frag[i]);
             (void)publish_dec_layers();
             return -1;
         }
-        if (i >= n_layers) free_layer(&g_vt.h_layers[i]);    /* a shorter backbone than before */
+        if (i < n_layers) (void)build_frag(&g_vt.h_frag[i], &g_vt.h_layers[i]);
+        if (i >= n_layers) { free_layer(&g_vt.h_layers[i]); free_frag(&g_vt.h_frag[i]); }   /* a shorter backbone than before */
     }
     if (publish_dec_layers()) return -1;
     if (g_vt.n_dec_layers != n_layers) { vt_set_error("tts_hip_upload_llm_weights: internal layer count"); return -1; }

@@ -16,6 +16,13 @@ void vt_launch_gemm(float *d_C, const uint16_t *d_Ahi, const uint16_t *d_Alo, co
 /* the same with the row pitch of C and the distance between planes given */
 void vt_launch_gemm_ex(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
                        const uint16_t *d_W, int M, int N, int K, int splits);
+/* The same product on the 128 x 256 tile kernel, which reads the weights in fragment order
+ * (vt_launch_frag_layout): N % 256 == 0, K % 64 == 0, an even number of 64-wide K steps per cut. */
+int vt_gemm_frag_shape_ok(int N, int K, int splits);
+void vt_launch_gemm_frag(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
+                         const uint16_t *d_Wf, int M, int N, int K, int splits);
+/* row-major bf16 W[N, K] -> the fragment-order copy (same size); N % 32 == 0, K % 64 == 0 */
+void vt_launch_frag_layout(uint16_t *d_Wf, const uint16_t *d_W, int N, int K);
 /* n even */
 void vt_launch_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_x, size_t n);
 /* rows of 3072: x += sum of planes (splits > 0), then planes of rmsnorm(x)*w (d_w != NULL) */

@@ -162,6 +162,236 @@ vt_gemm_mfma_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const ui
         }
 }
 
+/* ---- the same product, 128 x 256 tile, one workgroup per CU ---------------------------
+ * What bounds the 128 x 128 kernel above is the LDS: a 64 x 64 wave tile reads 24 KB of fragments
+ * (two activation planes and the weights) per 32 matrix instructions, three quarters of the LDS
+ * bandwidth of a CU with four waves at it, and every K step is a store -> barrier -> read chain.
+ * Here a wave owns 128 rows x 64 columns: the weights of its 64 columns are nobody else's in the
+ * workgroup, so they go from global memory straight into the B operand registers, and only the
+ * activation planes, which all four waves share, pass through the LDS: 8 KB of fragment reads per
+ * 16 matrix instructions, half the LDS bandwidth.  Two LDS stages: the planes of K step kt + 1
+ * are written while step kt is multiplied, one barrier per step; the global loads of step kt + 2
+ * are in flight meanwhile (every request unconditional, so the waits count exactly).  One
+ * workgroup of four waves per CU (a wave may then use the whole register file of its SIMD: 128
+ * accumulator registers, two sets of weight registers, two sets of fragments).
+ * The k order inside a matrix instruction is free as long as both operands agree: lane group g
+ * (lane / 32) takes k = 32 g + 8 ks .. + 8 of the 64-wide step in slice ks.
+ * A lane's operand is 8 consecutive k of ONE weight row, and the 32 lanes of a group are 32
+ * different rows: read from the row-major matrix, every load instruction touches 32 lines 6 KB
+ * apart, and the CU's address pipeline, not the matrix cores, sets the pace (measured: 434 against
+ * 518 TFLOP/s).  The backbone therefore keeps a second copy of its matrices in fragment order,
+ * written once at upload by vt_frag_layout_kernel: every load is then 1 KB of consecutive bytes.
+ * Needs N % 256 == 0, K % 64 == 0 and an even number of K steps per cut. */
+#define GW_TM 128
+#define GW_TN 256
+#define GW_PLANE (GW_TM * GM_ROWB)
+#define GW_STAGE (2 * GW_PLANE)
+#define GW_LDS (2 * GW_STAGE)
+
+struct gw_bregs { u32x4 v[2][4]; };          /* [column block][slice] */
+struct gw_aregs { u32x4 hi[4], lo[4]; };     /* staging: rows lr + 32 i */
+struct gw_frags { bf16x8 hi[4], lo[4]; };    /* one 16-wide slice of the 128 rows, both planes */
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+vt_gemm_wide_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const uint16_t *Wf,
+                    int M, int N, int K, int k_split, int m_tiles, int n_tiles, int ldc, size_t plane_stride) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int id = (int)blockIdx.x;
+    int mt, nt, sp;
+    if ((n_tiles & 7) == 0) {
+        /* slot id lands on XCD id % 8: keep the M tiles of one N tile there */
+        const int x = id & 7, q = id >> 3, r = q / m_tiles, npx = n_tiles >> 3;
+        mt = q % m_tiles;
+        nt = (r % npx) * 8 + x;
+        sp = r / npx;
+    } else {
+        const int r = id / m_tiles;
+        mt = id % m_tiles;
+        nt = r % n_tiles;
+        sp = r / n_tiles;
+    }
+    const int t = (int)threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int lr = t >> 3, lc = t & 7;               /* staging: row lr + 32 i, 16-byte chunk lc */
+    const int k0 = sp * k_split, tiles = k_split / GM_BK;
+
+    /* rows past M read row 0 of the tile again: their products land in accumulator rows that are
+     * never stored (the rows of a matrix instruction do not mix), so nothing has to be zeroed */
+    const uint16_t *pa[4], *pl[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int gm = mt * GW_TM + lr + 32 * i;
+        const size_t ao = (size_t)(gm < M ? gm : mt * GW_TM) * K + k0 + lc * 8;
+        pa[i] = Ahi + ao;
+        pl[i] = Alo + ao;
+    }
+    const size_t b_blk = (size_t)32 * K;
+
+    auto fetch_a = [&](gw_aregs &r, int kt) {
+        const int adv = (kt < tiles ? kt : tiles - 1) * GM_BK;      /* past the end: the last step once more */
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            r.hi[i] = gm_ld(pa[i] + adv);
+            r.lo[i] = gm_ld(pl[i] + adv);
+        }
+    };
+    /* weights in fragment order (vt_frag_layout_kernel): the 1 KB of slice j of K step ks of column block
+     * nb is contiguous, lane l's 16 bytes at 16 l */
+    const uint16_t *pf = Wf + (size_t)(nt * GW_TN + 64 * wave) * K + (size_t)k0 * 32 + lane * 8;
+    auto fetch_b_slice = [&](gw_bregs &r, int kt, int j) {
+        const int adv = (kt < tiles ? kt : tiles - 1) * 2048;
+        r.v[0][j] = gm_ld(pf + adv + 512 * j);
+        r.v[1][j] = gm_ld(pf + b_blk + adv + 512 * j);
+    };
+    const int st_off = lr * GM_ROWB + lc * 16;
+    auto store_a = [&](const gw_aregs &r, int stage) {
+        unsigned char *base = lds + stage * GW_STAGE + st_off;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            *reinterpret_cast<u32x4 *>(base + 32 * i * GM_ROWB) = r.hi[i];
+            *reinterpret_cast<u32x4 *>(base + GW_PLANE + 32 * i * GM_ROWB) = r.lo[i];
+        }
+    };
+
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[a][b][v] = 0.f;
+
+    const int fa_off = (lane & 31) * GM_ROWB + (lane >> 5) * 64;
+    auto read_frags = [&](gw_frags &f, int stage, int ks) {
+        const unsigned char *base = lds + stage * GW_STAGE + fa_off + ks * 16;
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            f.hi[a] = gm_frag(base + 32 * a * GM_ROWB);
+            f.lo[a] = gm_frag(base + GW_PLANE + 32 * a * GM_ROWB);
+        }
+    };
+    auto mma = [&](const gw_frags &f, const gw_bregs &rb, int ks) {
+        const bf16x8 b0 = __builtin_bit_cast(bf16x8, rb.v[0][ks]), b1 = __builtin_bit_cast(bf16x8, rb.v[1][ks]);
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            acc[a][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.lo[a], b0, acc[a][0], 0, 0, 0);
+            acc[a][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.lo[a], b1, acc[a][1], 0, 0, 0);
+        }
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            acc[a][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.hi[a], b0, acc[a][0], 0, 0, 0);
+            acc[a][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.hi[a], b1, acc[a][1], 0, 0, 0);
+        }
+    };
+
+    /* one K step: stage `stage` holds the planes of step kt and `cur` its weights; `ra` holds the
+     * planes of step kt + 1 (requested a step ago); f0 already holds the fragments of slice 0.  The
+     * fragments of a slice are requested in front of the sixteen matrix instructions of the slice
+     * before it, the weight registers of a slice are requested again (for step kt + 2) as soon as its
+     * instructions are out, and the scheduling barriers keep that order. */
+    gw_aregs ra;
+    gw_frags f0, f1;
+#define GW_FENCE() __builtin_amdgcn_sched_barrier(0)
+    auto step = [&](int kt, int stage, gw_bregs &cur) {
+        store_a(ra, stage ^ 1);
+        fetch_a(ra, kt + 2);
+        GW_FENCE();
+        read_frags(f1, stage, 1);
+        GW_FENCE();
+        mma(f0, cur, 0);
+        GW_FENCE();
+        fetch_b_slice(cur, kt + 2, 0);
+        read_frags(f0, stage, 2);
+        GW_FENCE();
+        mma(f1, cur, 1);
+        GW_FENCE();
+        fetch_b_slice(cur, kt + 2, 1);
+        read_frags(f1, stage, 3);
+        GW_FENCE();
+        mma(f0, cur, 2);
+        GW_FENCE();
+        fetch_b_slice(cur, kt + 2, 2);
+        GW_FENCE();
+        mma(f1, cur, 3);
+        GW_FENCE();
+        fetch_b_slice(cur, kt + 2, 3);
+        __syncthreads();
+        read_frags(f0, stage ^ 1, 0);
+        GW_FENCE();
+    };
+
+    gw_bregs b0, b1;
+    fetch_a(ra, 0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) fetch_b_slice(b0, 0, j);
+    store_a(ra, 0);
+    fetch_a(ra, 1);
+#pragma unroll
+    for (int j = 0; j < 4; j++) fetch_b_slice(b1, 1, j);
+    __syncthreads();
+    read_frags(f0, 0, 0);
+    for (int kt = 0; kt < tiles; kt += 2) {
+        step(kt, 0, b0);
+        step(kt + 1, 1, b1);
+    }
+#undef GW_FENCE
+
+    /* accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 */
+    float *Cs = C + (size_t)sp * plane_stride;
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const int col = nt * GW_TN + 64 * wave + 32 * b + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = mt * GW_TM + 32 * a + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                if (row < M) Cs[(size_t)row * ldc + col] = acc[a][b][v];
+            }
+        }
+}
+
+static int gm_blocks(size_t n);
+
+int vt_gemm_frag_shape_ok(int N, int K, int splits) {
+    return N % GW_TN == 0 && K % GM_BK == 0 && splits >= 1 && K % splits == 0 && (K / splits) % (2 * GM_BK) == 0;
+}
+
+void vt_launch_gemm_frag(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
+                         const uint16_t *d_Wf, int M, int N, int K, int splits) {
+    static int attr_set = 0;
+    if (!attr_set) {
+        if (vt_check(hipFuncSetAttribute((const void *)vt_gemm_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         GW_LDS), "product LDS size"))
+            return;
+        attr_set = 1;
+    }
+    const int m_tiles = (M + GW_TM - 1) / GW_TM, n_tiles = N / GW_TN;
+    hipLaunchKernelGGL(vt_gemm_wide_kernel, dim3(m_tiles * n_tiles * splits), dim3(256), GW_LDS, g_vt.stream,
+                       d_C, d_Ahi, d_Alo, d_Wf, M, N, K, K / splits, m_tiles, n_tiles, ldc, plane_stride);
+}
+
+/* Row-major W[N, K] (N % 32 == 0, K % 64 == 0) -> fragment order: the 16 bytes that lane l = 32 g + n % 32
+ * feeds to slice j of K step ks of column block nb = n / 32, i.e. W[n][64 ks + 32 g + 8 j .. + 8], go to
+ * 16-byte slot ((nb * K/64 + ks) * 4 + j) * 64 + l.  A block of 32 rows occupies the same 32 K elements
+ * in both layouts. */
+__global__ void vt_frag_layout_kernel(u32x4 *out, const uint16_t *W, size_t n_slots, int K) {
+    const int ksteps = K / GM_BK;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_slots; i += (size_t)gridDim.x * blockDim.x) {
+        const int l = (int)(i & 63), j = (int)((i >> 6) & 3);
+        const size_t blk = i >> 8;
+        const int ks = (int)(blk % ksteps);
+        const size_t nb = blk / ksteps;
+        const size_t n = nb * 32 + (l & 31);
+        out[i] = gm_ld(W + n * K + 64 * ks + 32 * (l >> 5) + 8 * j);
+    }
+}
+
+void vt_launch_frag_layout(uint16_t *d_Wf, const uint16_t *d_W, int N, int K) {
+    const size_t n_slots = (size_t)N * K / 8;
+    hipLaunchKernelGGL(vt_frag_layout_kernel, dim3(gm_blocks(n_slots)), dim3(256), 0, g_vt.stream, (u32x4 *)d_Wf, d_W,
+                       n_slots, K);
+}
+
 int vt_gemm_shape_ok(int M, int N, int K, int splits) {
     return M >= 1 && splits >= 1 && N % GM_TILE == 0 && K % splits == 0 && (K / splits) % GM_BK == 0;
 }

@@ -282,6 +282,10 @@ void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, c
 
 /* ---- backbone prefill ------------------------------------------------------------ */
 
+#ifndef VT_W13_TAIL_CUT
+#define VT_W13_TAIL_CUT 4
+#endif
+
 static int ew_blocks(size_t n) { size_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : b); }
 
 extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int start_pos, float *out_x) {
@@ -314,13 +318,28 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         const vt_layer_dev *L = &g_vt.h_layers[l];
         float *kc = g_hip.kv_cache_k_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
         float *vc = g_hip.kv_cache_v_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
-        vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
+        const vt_layer_frag *F = &g_vt.h_frag[l];
+        const bool frag = F->wqkv && F->wo && F->w13 && F->w2;
+        if (frag) vt_launch_gemm_frag(wide, VT_QKV_DIM, S * VT_QKV_DIM, hi, lo, F->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
+        else vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
         hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(ew_blocks(S * VT_QKV_DIM / 4)), dim3(256), 0, st,
                            wide, sp_qkv, S * VT_QKV_DIM, q, kc, vc, g_vt.d_rope, start_pos, seq_len);
         vt_launch_prefill_attention(NULL, hi, lo, q, VT_Q_DIM, kc, vc, seq_len, start_pos, VT_ATT_SCALE);
-        vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
+        if (frag) vt_launch_gemm_frag(part, VT_DIM, ps, hi, lo, F->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
+        else vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
         vt_launch_residual_norm_split(x, part, sp_wo, ps, L->ffn_norm, hi, lo, seq_len);
-        if (tail_cols) {
+        if (frag && m_tiles != 4) {
+            vt_launch_gemm_frag(wide, 2 * VT_FFN, 0, hi, lo, F->w13, seq_len, 2 * VT_FFN, VT_DIM, 1);
+            vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, 0, NULL, 0, 0);
+        } else if (frag) {
+            /* 4 M tiles x 72 N tiles of 256 columns are 288 workgroups for 256 CUs: the last 8 N tiles get
+             * their K cut in VT_W13_TAIL_CUT instead of running as a nearly empty second round */
+            const int tail = 8 * 256, main_cols = 2 * VT_FFN - tail;
+            vt_launch_gemm_frag(wide, 2 * VT_FFN, 0, hi, lo, F->w13, seq_len, main_cols, VT_DIM, 1);
+            vt_launch_gemm_frag(part, tail, S * tail, hi, lo, F->w13 + (size_t)main_cols * VT_DIM, seq_len, tail, VT_DIM,
+                                VT_W13_TAIL_CUT);
+            vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, main_cols, part, VT_W13_TAIL_CUT, S * tail);
+        } else if (tail_cols) {
             /* 4 M tiles x 144 N tiles are 576 workgroups for 512 slots: the last 16 N tiles get their
              * K cut in 4 instead of running as a nearly empty second round */
             const int main_cols = 2 * VT_FFN - tail_cols;
@@ -332,7 +351,8 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
             vt_launch_gemm(wide, hi, lo, L->w13, seq_len, 2 * VT_FFN, VT_DIM, 1);
             vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, 0, NULL, 0, 0);
         }
-        vt_launch_gemm(part, hi, lo, L->w2, seq_len, VT_DIM, VT_FFN, sp_w2);
+        if (frag) vt_launch_gemm_frag(part, VT_DIM, ps, hi, lo, F->w2, seq_len, VT_DIM, VT_FFN, sp_w2);
+        else vt_launch_gemm(part, hi, lo, L->w2, seq_len, VT_DIM, VT_FFN, sp_w2);
         const float *next_norm = l + 1 < g_vt.n_dec_layers ? g_vt.h_layers[l + 1].attn_norm : NULL;
         vt_launch_residual_norm_split(x, part, sp_w2, ps, next_norm, hi, lo, seq_len);
     }
@@ -378,12 +398,21 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
          * one layer they would be served from the memory-side cache */
         const vt_layer_dev *L = &g_vt.h_layers[(it + 2) % g_vt.n_dec_layers];
         const uint16_t *W[4] = {L->wqkv, L->wo, L->w13, L->w2};
-        if (which == 2) {                               /* as in the prefill: main part + K-cut tail */
+        const vt_layer_frag *F = &g_vt.h_frag[(it + 2) % g_vt.n_dec_layers];
+        const uint16_t *Wf[4] = {F->wqkv, F->wo, F->w13, F->w2};
+        const bool frag = F->wqkv && F->wo && F->w13 && F->w2;
+        if (which == 2 && frag) {                       /* as in the prefill: main part + K-cut tail */
+            const int tail = 8 * 256, main_cols = 2 * VT_FFN - tail;
+            vt_launch_gemm_frag(out, 2 * VT_FFN, 0, hi, lo, Wf[2], S, main_cols, VT_DIM, 1);
+            vt_launch_gemm_frag(out + (size_t)S * 2 * VT_FFN, tail, (size_t)S * tail, hi, lo,
+                                Wf[2] + (size_t)main_cols * VT_DIM, S, tail, VT_DIM, VT_W13_TAIL_CUT);
+        } else if (which == 2) {
             const int tail = 16 * 128, main_cols = 2 * VT_FFN - tail;
             vt_launch_gemm_ex(out, 2 * VT_FFN, 0, hi, lo, W[2], S, main_cols, VT_DIM, 1);
             vt_launch_gemm_ex(out + (size_t)S * 2 * VT_FFN, tail, (size_t)S * tail, hi, lo,
                               W[2] + (size_t)main_cols * VT_DIM, S, tail, VT_DIM, 4);
-        } else if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], SP[which]);
+        } else if (which < 4 && frag) vt_launch_gemm_frag(out, NN[which], (size_t)S * NN[which], hi, lo, Wf[which], S, NN[which], KK[which], SP[which]);
+        else if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], SP[which]);
         else vt_launch_prefill_attention(out, NULL, NULL, q, VT_Q_DIM, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu, S, 0, VT_ATT_SCALE);
     }
     if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;

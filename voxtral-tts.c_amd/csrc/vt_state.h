@@ -21,6 +21,10 @@
 #define VT_SEM_PADDED 8320
 #define VT_SEM_VALID_END 8194     /* 2 special + 8192 codes */
 
+/* Second copy of a backbone layer's four matrices, in the order the 128 x 256 tile product reads them
+ * (vt_launch_frag_layout); the decode step streams the row-major copy. */
+struct vt_layer_frag { uint16_t *wqkv, *wo, *w13, *w2; };
+
 struct vt_acoustic_dev {
     vt_layer_dev layers[TTS_HIP_AC_LAYERS];
     uint16_t *input_proj, *time_proj, *llm_proj, *semantic_out, *acoustic_out;
@@ -49,6 +53,7 @@ struct vt_state {
 
     /* backbone weights */
     vt_layer_dev h_layers[TTS_HIP_DEC_LAYERS];
+    vt_layer_frag h_frag[TTS_HIP_DEC_LAYERS];   /* the same matrices in the fragment order of the prefill product */
     vt_layer_dev *d_layers;
     float *d_dec_norm;
     uint16_t *d_tok_emb;
