@@ -21,6 +21,10 @@ void vt_launch_gemm_ex(float *d_C, int ldc, size_t plane_stride, const uint16_t 
 int vt_gemm_frag_shape_ok(int N, int K, int splits);
 void vt_launch_gemm_frag(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
                          const uint16_t *d_Wf, int M, int N, int K, int splits);
+/* the first n_main columns whole into d_C, the other n_tail columns with K cut in tail_splits into the
+ * planes d_tail [tail_splits][M, n_tail], in one launch (n_main, n_tail multiples of 256) */
+void vt_launch_gemm_frag_tail(float *d_C, int ldc, float *d_tail, const uint16_t *d_Ahi, const uint16_t *d_Alo,
+                              const uint16_t *d_Wf, int M, int n_main, int n_tail, int K, int tail_splits);
 /* row-major bf16 W[N, K] -> the fragment-order copy (same size); N % 32 == 0, K % 64 == 0 */
 void vt_launch_frag_layout(uint16_t *d_Wf, const uint16_t *d_W, int N, int K);
 /* n even */

@@ -192,18 +192,39 @@ struct gw_bregs { u32x4 v[2][4]; };          /* [column block][slice] */
 struct gw_aregs { u32x4 hi[4], lo[4]; };     /* staging: rows lr + 32 i */
 struct gw_frags { bf16x8 hi[4], lo[4]; };    /* one 16-wide slice of the 128 rows, both planes */
 
+/* A launch runs one or two sets of equal work items; workgroup i takes item i of each set in turn (a set
+ * may have fewer items than the grid).  The second set lets a product whose tile count is not a multiple
+ * of the CU count finish its last tiles as K cuts spread over all CUs inside the same launch. */
+struct gw_part {
+    float *C;                /* output of this set: `splits` planes, plane_stride floats apart, row pitch ldc */
+    const uint16_t *Wf;      /* fragment-order weights of the set's first column */
+    size_t plane_stride;
+    int ldc, n_tiles, splits, k_split;
+};
+struct gw_plan { gw_part part[2]; int n_parts; };
+
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-vt_gemm_wide_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const uint16_t *Wf,
-                    int M, int N, int K, int k_split, int m_tiles, int n_tiles, int ldc, size_t plane_stride) {
+vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int M, int K, int m_tiles) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int id = (int)blockIdx.x;
+  for (int pi = 0; pi < plan.n_parts; pi++) {
+    const gw_part &P = plan.part[pi];
+    const int n_tiles = P.n_tiles, k_split = P.k_split, ldc = P.ldc;
+    if (id >= m_tiles * n_tiles * P.splits) continue;
+    float *C = P.C;
+    const uint16_t *Wf = P.Wf;
+    const size_t plane_stride = P.plane_stride;
     int mt, nt, sp;
-    if ((n_tiles & 7) == 0) {
-        /* slot id lands on XCD id % 8: keep the M tiles of one N tile there */
-        const int x = id & 7, q = id >> 3, r = q / m_tiles, npx = n_tiles >> 3;
+    if (((n_tiles * P.splits) & 7) == 0) {
+        /* Slot id lands on XCD id % 8.  An XCD takes all M tiles of a run of consecutive (K cut, N tile)
+         * pairs: the M tiles of a pair share its weights, the N tiles of a K cut share the activation
+         * planes of that cut, and both then leave the memory side once per XCD instead of once per
+         * workgroup (the two slices are the same size: 128 rows x 4 bytes against 256 rows x 2 bytes). */
+        const int x = id & 7, q = id >> 3, per_xcd = (n_tiles * P.splits) >> 3;
+        const int ci = x * per_xcd + q / m_tiles;
         mt = q % m_tiles;
-        nt = (r % npx) * 8 + x;
-        sp = r / npx;
+        nt = ci % n_tiles;
+        sp = ci / n_tiles;
     } else {
         const int r = id / m_tiles;
         mt = id % m_tiles;
@@ -348,6 +369,8 @@ vt_gemm_wide_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const ui
                 if (row < M) Cs[(size_t)row * ldc + col] = acc[a][b][v];
             }
         }
+    __syncthreads();                 /* the next item refills the LDS stages */
+  }
 }
 
 static int gm_blocks(size_t n);
@@ -356,18 +379,43 @@ int vt_gemm_frag_shape_ok(int N, int K, int splits) {
     return N % GW_TN == 0 && K % GM_BK == 0 && splits >= 1 && K % splits == 0 && (K / splits) % (2 * GM_BK) == 0;
 }
 
-void vt_launch_gemm_frag(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
-                         const uint16_t *d_Wf, int M, int N, int K, int splits) {
+static int gw_ready(void) {
     static int attr_set = 0;
     if (!attr_set) {
         if (vt_check(hipFuncSetAttribute((const void *)vt_gemm_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                          GW_LDS), "product LDS size"))
-            return;
+            return 0;
         attr_set = 1;
     }
-    const int m_tiles = (M + GW_TM - 1) / GW_TM, n_tiles = N / GW_TN;
-    hipLaunchKernelGGL(vt_gemm_wide_kernel, dim3(m_tiles * n_tiles * splits), dim3(256), GW_LDS, g_vt.stream,
-                       d_C, d_Ahi, d_Alo, d_Wf, M, N, K, K / splits, m_tiles, n_tiles, ldc, plane_stride);
+    return 1;
+}
+
+void vt_launch_gemm_frag(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
+                         const uint16_t *d_Wf, int M, int N, int K, int splits) {
+    if (!gw_ready()) return;
+    const int m_tiles = (M + GW_TM - 1) / GW_TM;
+    gw_plan plan = {};
+    plan.n_parts = 1;
+    plan.part[0] = gw_part{d_C, d_Wf, plane_stride, ldc, N / GW_TN, splits, K / splits};
+    hipLaunchKernelGGL(vt_gemm_wide_kernel, dim3(m_tiles * (N / GW_TN) * splits), dim3(256), GW_LDS, g_vt.stream,
+                       plan, d_Ahi, d_Alo, M, K, m_tiles);
+}
+
+/* One launch for a product whose columns are cut in two sets: the first n_main columns whole (into d_C, row
+ * pitch ldc), the other n_tail columns with K cut in `tail_splits` (into d_tail, `tail_splits` planes of
+ * [M, n_tail]).  Every workgroup takes one item of each set. */
+void vt_launch_gemm_frag_tail(float *d_C, int ldc, float *d_tail, const uint16_t *d_Ahi, const uint16_t *d_Alo,
+                              const uint16_t *d_Wf, int M, int n_main, int n_tail, int K, int tail_splits) {
+    if (!gw_ready()) return;
+    const int m_tiles = (M + GW_TM - 1) / GW_TM;
+    gw_plan plan = {};
+    plan.n_parts = 2;
+    plan.part[0] = gw_part{d_C, d_Wf, 0, ldc, n_main / GW_TN, 1, K};
+    plan.part[1] = gw_part{d_tail, d_Wf + (size_t)n_main * K, (size_t)M * n_tail, n_tail, n_tail / GW_TN, tail_splits,
+                           K / tail_splits};
+    const int items0 = m_tiles * (n_main / GW_TN), items1 = m_tiles * (n_tail / GW_TN) * tail_splits;
+    hipLaunchKernelGGL(vt_gemm_wide_kernel, dim3(items0 > items1 ? items0 : items1), dim3(256), GW_LDS, g_vt.stream,
+                       plan, d_Ahi, d_Alo, M, K, m_tiles);
 }
 
 /* Row-major W[N, K] (N % 32 == 0, K % 64 == 0) -> fragment order: the 16 bytes that lane l = 32 g + n % 32

@@ -332,12 +332,11 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
             vt_launch_gemm_frag(wide, 2 * VT_FFN, 0, hi, lo, F->w13, seq_len, 2 * VT_FFN, VT_DIM, 1);
             vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, 0, NULL, 0, 0);
         } else if (frag) {
-            /* 4 M tiles x 72 N tiles of 256 columns are 288 workgroups for 256 CUs: the last 8 N tiles get
-             * their K cut in VT_W13_TAIL_CUT instead of running as a nearly empty second round */
+            /* 4 M tiles x 72 N tiles of 256 columns are 288 items for 256 CUs: the last 8 N tiles get their K cut
+             * in VT_W13_TAIL_CUT and every workgroup takes one of those cuts after its whole tile, in the same
+             * launch, instead of 32 workgroups running a second round alone */
             const int tail = 8 * 256, main_cols = 2 * VT_FFN - tail;
-            vt_launch_gemm_frag(wide, 2 * VT_FFN, 0, hi, lo, F->w13, seq_len, main_cols, VT_DIM, 1);
-            vt_launch_gemm_frag(part, tail, S * tail, hi, lo, F->w13 + (size_t)main_cols * VT_DIM, seq_len, tail, VT_DIM,
-                                VT_W13_TAIL_CUT);
+            vt_launch_gemm_frag_tail(wide, 2 * VT_FFN, part, hi, lo, F->w13, seq_len, main_cols, tail, VT_DIM, VT_W13_TAIL_CUT);
             vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, main_cols, part, VT_W13_TAIL_CUT, S * tail);
         } else if (tail_cols) {
             /* 4 M tiles x 144 N tiles are 576 workgroups for 512 slots: the last 16 N tiles get their
@@ -403,9 +402,8 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
         const bool frag = F->wqkv && F->wo && F->w13 && F->w2;
         if (which == 2 && frag) {                       /* as in the prefill: main part + K-cut tail */
             const int tail = 8 * 256, main_cols = 2 * VT_FFN - tail;
-            vt_launch_gemm_frag(out, 2 * VT_FFN, 0, hi, lo, Wf[2], S, main_cols, VT_DIM, 1);
-            vt_launch_gemm_frag(out + (size_t)S * 2 * VT_FFN, tail, (size_t)S * tail, hi, lo,
-                                Wf[2] + (size_t)main_cols * VT_DIM, S, tail, VT_DIM, VT_W13_TAIL_CUT);
+            vt_launch_gemm_frag_tail(out, 2 * VT_FFN, out + (size_t)S * 2 * VT_FFN, hi, lo, Wf[2], S, main_cols, tail, VT_DIM,
+                                     VT_W13_TAIL_CUT);
         } else if (which == 2) {
             const int tail = 16 * 128, main_cols = 2 * VT_FFN - tail;
             vt_launch_gemm_ex(out, 2 * VT_FFN, 0, hi, lo, W[2], S, main_cols, VT_DIM, 1);
