@@ -175,7 +175,7 @@ __device__ __forceinline__ vt_rows vt_split_rows(int n_rows, int align, int k_pe
  * acknowledgement of the hand-over stores that the barrier waits for. */
 enum { VT_PART_ALL = 0, VT_PART_HEAD = 1, VT_PART_TAIL = 2 };
 #ifndef VT_HEAD_SLOTS
-#define VT_HEAD_SLOTS 6        /* ring slots (KB per wave) requested ahead of the hand-over */
+#define VT_HEAD_SLOTS 5        /* ring slots (KB per wave) requested ahead of the hand-over (4 / 5 / 6 / 7 / 8: 1.200 / 1.190 / 1.194 / 1.200 / 1.222 ms/frame) */
 #endif
 
 /* Only the ring slots [slot_lo, slot_hi) are requested: the output projection leaves the last 6

@@ -175,7 +175,9 @@ struct vt_grid_sync {
  * channels); a workgroup writes all copies and polls copy blockIdx % VT_FLAG_COPIES: the polls
  * of 256 workgroups are coherent loads served by the memory side, and spread over the copies
  * they do not queue on one channel. */
+#ifndef VT_FLAG_COPIES
 #define VT_FLAG_COPIES 8
+#endif
 #define VT_FLAG_STRIDE 16384
 /* Words between the flags of two workgroups: partial writes to one 64-byte line are served one
  * after another by the memory side (about 60 ns each, measured: 256 workgroups writing 16 flags to
@@ -185,8 +187,17 @@ struct vt_grid_sync {
 #define VT_FLAG_PAD 4
 #endif
 #define VT_FLAG_LOADS 4           /* flags a lane polls: grids of up to 256 workgroups */
+#define VT_FLAG_ABORT_AT 8192     /* word of a copy that says "a workgroup has given up" (one word read by 256
+                                   * workgroups at every poll would be a queue of its own) */
+/* Polls in flight per workgroup, and the pause (in units of 64 clocks) in front of a repeated poll.
+ * The polls of 256 workgroups are traffic on the memory side themselves: measured on the whole-step
+ * kernel, ms/frame with 4 / 3 / 2 / 1 polls in flight: 1.219 / 1.209 / 1.205 / 1.195, and 1.190
+ * with one poll and a pause of 2-12 units. */
 #ifndef VT_POLL_DEPTH
-#define VT_POLL_DEPTH 2
+#define VT_POLL_DEPTH 1
+#endif
+#ifndef VT_POLL_SLEEP
+#define VT_POLL_SLEEP 4
 #endif
 
 __device__ __forceinline__ void vt_barrier_arrive(vt_grid_sync &gs) {
@@ -201,9 +212,7 @@ __device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag)
         const unsigned *mine = gs.flags + (blockIdx.x % VT_FLAG_COPIES) * VT_FLAG_STRIDE;
         const unsigned long long t0 = wall_clock64();
         int ok = 1;
-        /* VT_POLL_DEPTH polls are kept in flight, so the release is seen a fraction of a memory
-         * latency after it could be.  A lane reads the flags lane, lane + 64, ... (the last one
-         * again where the grid has fewer). */
+        /* A lane reads the flags lane, lane + 64, ... (the last one again where the grid has fewer). */
         const int lane = (int)threadIdx.x;
         unsigned f[VT_POLL_DEPTH][VT_FLAG_LOADS];
 #pragma unroll
@@ -213,7 +222,7 @@ __device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag)
         bool released = false;
         while (!released) {
             /* the abort flag travels with the flags: one round trip per poll, not two */
-            const int aborted = __hip_atomic_load(gs.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int aborted = (int)vt_ldc_u32(mine + VT_FLAG_ABORT_AT);
 #pragma unroll
             for (int d = 0; d < VT_POLL_DEPTH; d++) {
                 if (!released) {
@@ -222,6 +231,7 @@ __device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag)
                     for (int k = 0; k < VT_FLAG_LOADS; k++) done &= (int)(f[d][k] - gs.epoch) >= 0;
                     released = __all(done);
                     if (!released) {
+                        if (VT_POLL_SLEEP > 0) __builtin_amdgcn_s_sleep(VT_POLL_SLEEP);
 #pragma unroll
                         for (int k = 0; k < VT_FLAG_LOADS; k++)
                             f[d][k] = vt_ldc_u32(mine + min(lane + VT_WAVE * k, G - 1) * VT_FLAG_PAD);
@@ -234,10 +244,12 @@ __device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag)
             }
         }
         ok = __all(ok);
-        if (threadIdx.x == 0) {
-            if (!ok) __hip_atomic_store(gs.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            *lds_flag = ok;
+        if (!ok) {
+            /* the host reads abort_flag; the other workgroups read the copy that travels with their flags */
+            if (threadIdx.x == 0) __hip_atomic_store(gs.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (threadIdx.x < VT_FLAG_COPIES) vt_stc_u32(gs.flags + threadIdx.x * VT_FLAG_STRIDE + VT_FLAG_ABORT_AT, 1u);
         }
+        if (threadIdx.x == 0) *lds_flag = ok;
     }
     __syncthreads();
     gs.epoch += 1u;
