@@ -304,40 +304,52 @@ vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int 
         }
     };
 
-    /* one K step: stage `stage` holds the planes of step kt and `cur` its weights; `ra` holds the
-     * planes of step kt + 1 (requested a step ago); f0 already holds the fragments of slice 0.  The
-     * fragments of a slice are requested in front of the sixteen matrix instructions of the slice
-     * before it, the weight registers of a slice are requested again (for step kt + 2) as soon as its
-     * instructions are out, and the scheduling barriers keep that order. */
+    /* One K step: stage `stage` holds the planes of step kt and `cur` its weights; `ra` holds the planes
+     * of step kt + 1 (requested a step ago); f0 already holds the fragments of slice 0.  Four regions of
+     * sixteen matrix instructions each; the other instructions of a region (the fragment reads of the next
+     * slice, in the first region also the LDS stores of step kt + 1 and the plane requests of step kt + 2,
+     * in the others the two weight requests that refill the slice just used) are dealt out between the
+     * matrix instructions, one after every second, so that the matrix pipe never waits for a block of
+     * them to issue.  The step's one barrier stands in front of the last region: by then every wave has
+     * issued (and waited for) its stores into the other stage and its last reads of this one, so the first
+     * fragments of step kt + 1 are read under the last sixteen matrix instructions of step kt. */
     gw_aregs ra;
     gw_frags f0, f1;
 #define GW_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define GW_MFMA2() __builtin_amdgcn_sched_group_barrier(0x008, 2, 0)
+#define GW_DSR1() __builtin_amdgcn_sched_group_barrier(0x100, 1, 0)
+#define GW_DSW1() __builtin_amdgcn_sched_group_barrier(0x200, 1, 0)
+#define GW_VMR1() __builtin_amdgcn_sched_group_barrier(0x020, 1, 0)
     auto step = [&](int kt, int stage, gw_bregs &cur) {
+        GW_FENCE();
         store_a(ra, stage ^ 1);
         fetch_a(ra, kt + 2);
-        GW_FENCE();
         read_frags(f1, stage, 1);
-        GW_FENCE();
         mma(f0, cur, 0);
+#pragma unroll
+        for (int i = 0; i < 8; i++) { GW_MFMA2(); GW_DSR1(); GW_DSW1(); GW_VMR1(); }
         GW_FENCE();
         fetch_b_slice(cur, kt + 2, 0);
         read_frags(f0, stage, 2);
-        GW_FENCE();
         mma(f1, cur, 1);
+#pragma unroll
+        for (int i = 0; i < 8; i++) { GW_MFMA2(); GW_DSR1(); if (i < 2) GW_VMR1(); }
         GW_FENCE();
         fetch_b_slice(cur, kt + 2, 1);
         read_frags(f1, stage, 3);
-        GW_FENCE();
         mma(f0, cur, 2);
+#pragma unroll
+        for (int i = 0; i < 8; i++) { GW_MFMA2(); GW_DSR1(); if (i < 2) GW_VMR1(); }
+        GW_FENCE();
+        __syncthreads();
         GW_FENCE();
         fetch_b_slice(cur, kt + 2, 2);
-        GW_FENCE();
+        read_frags(f0, stage ^ 1, 0);
         mma(f1, cur, 3);
+#pragma unroll
+        for (int i = 0; i < 8; i++) { GW_MFMA2(); GW_DSR1(); if (i < 2) GW_VMR1(); }
         GW_FENCE();
         fetch_b_slice(cur, kt + 2, 3);
-        __syncthreads();
-        read_frags(f0, stage ^ 1, 0);
-        GW_FENCE();
     };
 
     gw_bregs b0, b1;
@@ -354,6 +366,10 @@ vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int 
         step(kt, 0, b0);
         step(kt + 1, 1, b1);
     }
+#undef GW_MFMA2
+#undef GW_DSR1
+#undef GW_DSW1
+#undef GW_VMR1
 #undef GW_FENCE
 
     /* accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 */
