@@ -41,16 +41,21 @@ __device__ __forceinline__ void vt_tr(int &n) {
 #define VT_TR(n) ((void)0)
 #endif
 
-template <class F>
-__device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between, int &tn) {
+template <class F, class W>
+__device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between, int &tn, W wait) {
     VT_TR(tn);                      /* body done */
     vt_barrier_arrive(gs);
     VT_TR(tn);                      /* arrived */
     between();
     VT_TR(tn);                      /* prefetch requested */
-    const bool ok = vt_barrier_wait(gs, flag);
+    const bool ok = wait();
     VT_TR(tn);                      /* released */
     return ok;
+}
+
+template <class F>
+__device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between, int &tn) {
+    return vt_barrier_then(gs, flag, between, tn, [&] { return vt_barrier_wait(gs, flag); });
 }
 
 __global__ void __launch_bounds__(VT_STEP_THREADS)
@@ -69,6 +74,20 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
     /* scalars of the whole step: who runs the attention, and whether enough workgroups are left over */
     const int att_busy = __builtin_amdgcn_readfirstlane(vt_attn_busy(a));
     const bool l2_prefetch = 4 * att_busy <= 3 * (int)gridDim.x;
+    /* The two hand-overs around the attention are narrow.  Into it: a workgroup of the direct schedule
+     * reads the q rows of one head and the new K and V rows of one kv head, which some 20 workgroups
+     * wrote, and the workgroups without a share of the attention read nothing.  Out of it: everybody
+     * reads what the att_busy attention workgroups wrote.  Those have, between them, waited for every
+     * workgroup that owns q|k|v rows, so behind the second hand-over nobody still reads the residual
+     * stream that the output projection is about to overwrite. */
+    const bool att_direct = vt_attn_is_direct(a);
+    auto wait_qkv = [&]() -> bool {
+        if (!att_direct) return vt_barrier_wait(gs, &s_flag);
+        if ((int)blockIdx.x >= att_busy) { vt_barrier_pass(gs); return true; }
+        const int lane = (int)threadIdx.x & (VT_WAVE - 1);
+        return vt_barrier_wait_on(gs, &s_flag, 1, [&](int) { return vt_attn_producer((int)blockIdx.x, lane); });
+    };
+    auto wait_attn = [&]() -> bool { return vt_barrier_wait_first(gs, &s_flag, att_busy); };
     for (int l = 0; l < a.n_layers; l++) {
         const vt_layer_dev L = a.layers[l];
         /* the next phase's first row is requested as soon as the ring is free, the other rows
@@ -76,7 +95,7 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
          * busy from the end of one phase's arithmetic to the start of the next one's */
         const bool more = l + 1 < a.n_layers;
         vt_qkv_body(ring, L, a, l, x_in, lds, [&] { vt_wo_prefetch(ring, L, VT_PART_HEAD); });
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_wo_prefetch(ring, L, VT_PART_TAIL); }, tn)) return;
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_wo_prefetch(ring, L, VT_PART_TAIL); }, tn, wait_qkv)) return;
         vt_attn_phase(a, l, lds);
         /* with 3 rows per wave the output projection leaves the ring slots from VT_WO_SLOTS on
          * free: the gate|up rows that go there are requested a phase early */
@@ -90,7 +109,7 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
                     vt_w13_l2_prefetch(L, att_busy);
                     if (more && vt_attn_is_direct(a)) vt_kv_l2_prefetch(a, l + 1, att_busy);
                 }
-            }, tn))
+            }, tn, wait_attn))
             return;
         vt_wo_body(ring, L, a, x_in, lds, [&] { vt_w13_prefetch(ring, L, VT_PART_HEAD, 0, wo_slots); });
         if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L, VT_PART_TAIL, 0, wo_slots); }, tn))

@@ -479,6 +479,25 @@ __device__ __forceinline__ void vt_attn_direct(const vt_step_args &a, int layer,
     }
 }
 
+/* The i-th of the workgroups whose q|k|v rows attention workgroup `wg` of the direct schedule reads
+ * (past the last one: the first again): the owners of the 128 rows of its query head and of the new K
+ * and V rows of its kv head, in the row split of vt_qkv_rows().  At most 7 + 7 + 7 on 256 workgroups. */
+__device__ __forceinline__ int vt_attn_producer(int wg, int i) {
+    const int G = (int)gridDim.x;
+    int per = (VT_QKV_DIM + G - 1) / G;
+    per = (per + 1) / 2 * 2;
+    const int kvh = wg % VT_KV_HEADS, head = kvh * 4 + ((wg / VT_KV_HEADS) & 3);
+    const int first[3] = {head * VT_HEAD_DIM, VT_Q_DIM + kvh * VT_HEAD_DIM, VT_Q_DIM + VT_KV_DIM + kvh * VT_HEAD_DIM};
+    int j = i;
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        const int w0 = first[k] / per, n = (first[k] + VT_HEAD_DIM - 1) / per - w0 + 1;
+        if (j < n) return w0 + j;
+        j -= n;
+    }
+    return first[0] / per;
+}
+
 /* The output projection's input vector into LDS: the attention output as it stands, or the
  * combination of the NS partials per head the split schedule left (online-softmax algebra of
  * voxtral_tts_kernels.c:426-462, parts in ascending order). */

@@ -206,19 +206,24 @@ __device__ __forceinline__ void vt_barrier_arrive(vt_grid_sync &gs) {
     if (threadIdx.x < VT_FLAG_COPIES) vt_stc_u32(gs.flags + threadIdx.x * VT_FLAG_STRIDE + blockIdx.x * VT_FLAG_PAD, gs.epoch);
 }
 
-__device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag) {
+/* Wait until the workgroups idx(0) .. idx(nloads - 1) of every lane have announced the current
+ * barrier (the first wave polls; a lane with fewer workgroups to watch names one of them again).
+ * A hand-over that only some workgroups feed needs only their flags: fewer lines per poll, and
+ * nobody waits for a straggler whose results it does not read. */
+template <class IDX>
+__device__ __forceinline__ bool vt_barrier_wait_on(vt_grid_sync &gs, int *lds_flag, int nloads, IDX idx) {
     if (threadIdx.x < VT_WAVE) {
-        const int G = (int)gridDim.x;
         const unsigned *mine = gs.flags + (blockIdx.x % VT_FLAG_COPIES) * VT_FLAG_STRIDE;
         const unsigned long long t0 = wall_clock64();
         int ok = 1;
-        /* A lane reads the flags lane, lane + 64, ... (the last one again where the grid has fewer). */
-        const int lane = (int)threadIdx.x;
         unsigned f[VT_POLL_DEPTH][VT_FLAG_LOADS];
+        int at[VT_FLAG_LOADS];
+#pragma unroll
+        for (int k = 0; k < VT_FLAG_LOADS; k++) at[k] = idx(k < nloads ? k : 0) * VT_FLAG_PAD;
 #pragma unroll
         for (int d = 0; d < VT_POLL_DEPTH; d++)
 #pragma unroll
-            for (int k = 0; k < VT_FLAG_LOADS; k++) f[d][k] = vt_ldc_u32(mine + min(lane + VT_WAVE * k, G - 1) * VT_FLAG_PAD);
+            for (int k = 0; k < VT_FLAG_LOADS; k++) f[d][k] = k < nloads ? vt_ldc_u32(mine + at[k]) : gs.epoch;
         bool released = false;
         while (!released) {
             /* the abort flag travels with the flags: one round trip per poll, not two */
@@ -234,7 +239,7 @@ __device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag)
                         if (VT_POLL_SLEEP > 0) __builtin_amdgcn_s_sleep(VT_POLL_SLEEP);
 #pragma unroll
                         for (int k = 0; k < VT_FLAG_LOADS; k++)
-                            f[d][k] = vt_ldc_u32(mine + min(lane + VT_WAVE * k, G - 1) * VT_FLAG_PAD);
+                            if (k < nloads) f[d][k] = vt_ldc_u32(mine + at[k]);
                     }
                 }
             }
@@ -255,5 +260,20 @@ __device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag)
     gs.epoch += 1u;
     return *lds_flag != 0;
 }
+
+/* every workgroup: a lane reads the flags lane, lane + 64, ... (the last one again where the grid has fewer) */
+__device__ __forceinline__ bool vt_barrier_wait(vt_grid_sync &gs, int *lds_flag) {
+    const int G = (int)gridDim.x, lane = (int)threadIdx.x & (VT_WAVE - 1);
+    return vt_barrier_wait_on(gs, lds_flag, VT_FLAG_LOADS, [&](int k) { return min(lane + VT_WAVE * k, G - 1); });
+}
+
+/* the workgroups 0 .. n - 1 */
+__device__ __forceinline__ bool vt_barrier_wait_first(vt_grid_sync &gs, int *lds_flag, int n) {
+    const int lane = (int)threadIdx.x & (VT_WAVE - 1);
+    return vt_barrier_wait_on(gs, lds_flag, (n + VT_WAVE - 1) / VT_WAVE, [&](int k) { return min(lane + VT_WAVE * k, n - 1); });
+}
+
+/* A workgroup that reads nothing of what this hand-over passes on: it has announced itself and goes on. */
+__device__ __forceinline__ void vt_barrier_pass(vt_grid_sync &gs) { gs.epoch += 1u; }
 
 #endif /* VT_DEVICE_H */
