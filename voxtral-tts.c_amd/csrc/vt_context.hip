@@ -165,7 +165,7 @@ static int build_frag(vt_layer_frag *g, const vt_layer_dev *l) {
         {&g->w13, l->w13, 2 * VT_FFN, VT_DIM}, {&g->w2, l->w2, VT_DIM, VT_FFN}};
     for (int i = 0; i < 4; i++) {
         if (!(*m[i].dst = (uint16_t *)vt_dev_alloc((size_t)m[i].n * m[i].k * 2))) { free_frag(g); return -1; }
-        vt_launch_frag_layout(*m[i].dst, m[i].src, m[i].n, m[i].k);
+        vt_launch_frag_layout(*m[i].dst, m[i].src, m[i].n, m[i].k, i == 2);      /* gate|up: paired */
     }
     if (vt_check(hipGetLastError(), "fragment layout launch") || vt_check(hipStreamSynchronize(g_vt.stream), "fragment layout")) {
         free_frag(g);

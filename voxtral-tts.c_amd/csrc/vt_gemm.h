@@ -21,12 +21,18 @@ void vt_launch_gemm_ex(float *d_C, int ldc, size_t plane_stride, const uint16_t 
 int vt_gemm_frag_shape_ok(int N, int K, int splits);
 void vt_launch_gemm_frag(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
                          const uint16_t *d_Wf, int M, int N, int K, int splits);
-/* the first n_main columns whole into d_C, the other n_tail columns with K cut in tail_splits into the
- * planes d_tail [tail_splits][M, n_tail], in one launch (n_main, n_tail multiples of 256) */
-void vt_launch_gemm_frag_tail(float *d_C, int ldc, float *d_tail, const uint16_t *d_Ahi, const uint16_t *d_Alo,
-                              const uint16_t *d_Wf, int M, int n_main, int n_tail, int K, int tail_splits);
-/* row-major bf16 W[N, K] -> the fragment-order copy (same size); N % 32 == 0, K % 64 == 0 */
-void vt_launch_frag_layout(uint16_t *d_Wf, const uint16_t *d_W, int N, int K);
+/* row-major bf16 W[N, K] -> the fragment-order copy (same size); N % 32 == 0, K % 64 == 0.  pair: W holds
+ * (gate, up) rows interleaved and every 64 fragment columns become 32 gates followed by their 32 ups
+ * (N % 64 == 0), the order vt_launch_gemm_frag_swiglu expects. */
+void vt_launch_frag_layout(uint16_t *d_Wf, const uint16_t *d_W, int N, int K, int pair);
+/* gate|up product on paired weights with SiLU(gate) * up as its epilogue: the first n_main columns leave the
+ * planes d_hhi / d_hlo [M, ldh] (n_main / 2 columns); the other n_tail columns (may be 0) have K cut in
+ * tail_splits and leave fp32 planes d_tail [tail_splits][M, n_tail] for vt_launch_swiglu_pair_tail */
+void vt_launch_gemm_frag_swiglu(uint16_t *d_hhi, uint16_t *d_hlo, int ldh, float *d_tail, const uint16_t *d_Ahi,
+                                const uint16_t *d_Alo, const uint16_t *d_Wf, int M, int n_main, int n_tail, int K,
+                                int tail_splits);
+void vt_launch_swiglu_pair_tail(uint16_t *d_hi, uint16_t *d_lo, int ldh, int h_col0, const float *d_tail, int planes,
+                                size_t stride, int rows, int tw);
 /* n even */
 void vt_launch_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_x, size_t n);
 /* rows of 3072: x += sum of planes (splits > 0), then planes of rmsnorm(x)*w (d_w != NULL) */

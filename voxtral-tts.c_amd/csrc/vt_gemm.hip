@@ -200,6 +200,10 @@ struct gw_part {
     const uint16_t *Wf;      /* fragment-order weights of the set's first column */
     size_t plane_stride;
     int ldc, n_tiles, splits, k_split;
+    /* gate|up product in the paired column order (vt_launch_frag_layout with pair = 1): instead of C, the
+     * (hi, lo) planes of SiLU(gate) * up, row pitch ldh; the set's first column is h column h_col0 */
+    uint16_t *h_hi, *h_lo;
+    int ldh, h_col0;
 };
 struct gw_plan { gw_part part[2]; int n_parts; };
 
@@ -373,6 +377,25 @@ vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int 
 #undef GW_FENCE
 
     /* accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 */
+    if (P.h_hi) {
+        /* a wave's two column blocks are the gates and the ups of the same 32 h columns
+         * (voxtral_tts_llm.c:346-350) */
+        const int hc = P.h_col0 + nt * (GW_TN / 2) + 32 * wave + (lane & 31);
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = mt * GW_TM + 32 * a + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                const float g = acc[a][0][v], u = acc[a][1][v];
+                const float h = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
+                unsigned sh, sl;
+                vt_split_planes2(h, 0.f, sh, sl);
+                if (row < M) {
+                    P.h_hi[(size_t)row * P.ldh + hc] = (uint16_t)sh;
+                    P.h_lo[(size_t)row * P.ldh + hc] = (uint16_t)sl;
+                }
+            }
+    } else {
     float *Cs = C + (size_t)sp * plane_stride;
 #pragma unroll
     for (int a = 0; a < 4; a++)
@@ -385,6 +408,7 @@ vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int 
                 if (row < M) Cs[(size_t)row * ldc + col] = acc[a][b][v];
             }
         }
+    }
     __syncthreads();                 /* the next item refills the LDS stages */
   }
 }
@@ -412,48 +436,57 @@ void vt_launch_gemm_frag(float *d_C, int ldc, size_t plane_stride, const uint16_
     const int m_tiles = (M + GW_TM - 1) / GW_TM;
     gw_plan plan = {};
     plan.n_parts = 1;
-    plan.part[0] = gw_part{d_C, d_Wf, plane_stride, ldc, N / GW_TN, splits, K / splits};
+    plan.part[0] = gw_part{d_C, d_Wf, plane_stride, ldc, N / GW_TN, splits, K / splits, NULL, NULL, 0, 0};
     hipLaunchKernelGGL(vt_gemm_wide_kernel, dim3(m_tiles * (N / GW_TN) * splits), dim3(256), GW_LDS, g_vt.stream,
                        plan, d_Ahi, d_Alo, M, K, m_tiles);
 }
 
-/* One launch for a product whose columns are cut in two sets: the first n_main columns whole (into d_C, row
- * pitch ldc), the other n_tail columns with K cut in `tail_splits` (into d_tail, `tail_splits` planes of
- * [M, n_tail]).  Every workgroup takes one item of each set. */
-void vt_launch_gemm_frag_tail(float *d_C, int ldc, float *d_tail, const uint16_t *d_Ahi, const uint16_t *d_Alo,
-                              const uint16_t *d_Wf, int M, int n_main, int n_tail, int K, int tail_splits) {
+/* gate|up product with the SiLU(gate) * up epilogue (weights in the paired fragment order): the first n_main
+ * columns go straight into the planes d_hhi / d_hlo [M, ldh]; the other n_tail columns (0: none) have K cut
+ * in tail_splits and leave fp32 planes d_tail [tail_splits][M, n_tail] in the paired column order, which
+ * vt_launch_swiglu_pair_tail turns into the last n_tail / 2 plane columns.  One launch. */
+void vt_launch_gemm_frag_swiglu(uint16_t *d_hhi, uint16_t *d_hlo, int ldh, float *d_tail, const uint16_t *d_Ahi,
+                                const uint16_t *d_Alo, const uint16_t *d_Wf, int M, int n_main, int n_tail, int K,
+                                int tail_splits) {
     if (!gw_ready()) return;
     const int m_tiles = (M + GW_TM - 1) / GW_TM;
     gw_plan plan = {};
-    plan.n_parts = 2;
-    plan.part[0] = gw_part{d_C, d_Wf, 0, ldc, n_main / GW_TN, 1, K};
-    plan.part[1] = gw_part{d_tail, d_Wf + (size_t)n_main * K, (size_t)M * n_tail, n_tail, n_tail / GW_TN, tail_splits,
-                           K / tail_splits};
-    const int items0 = m_tiles * (n_main / GW_TN), items1 = m_tiles * (n_tail / GW_TN) * tail_splits;
-    hipLaunchKernelGGL(vt_gemm_wide_kernel, dim3(items0 > items1 ? items0 : items1), dim3(256), GW_LDS, g_vt.stream,
-                       plan, d_Ahi, d_Alo, M, K, m_tiles);
+    plan.n_parts = n_tail > 0 ? 2 : 1;
+    plan.part[0] = gw_part{NULL, d_Wf, 0, 0, n_main / GW_TN, 1, K, d_hhi, d_hlo, ldh, 0};
+    int items = m_tiles * (n_main / GW_TN);
+    if (n_tail > 0) {
+        plan.part[1] = gw_part{d_tail, d_Wf + (size_t)n_main * K, (size_t)M * n_tail, n_tail, n_tail / GW_TN, tail_splits,
+                               K / tail_splits, NULL, NULL, 0, 0};
+        const int items1 = m_tiles * (n_tail / GW_TN) * tail_splits;
+        if (items1 > items) items = items1;
+    }
+    hipLaunchKernelGGL(vt_gemm_wide_kernel, dim3(items), dim3(256), GW_LDS, g_vt.stream, plan, d_Ahi, d_Alo, M, K, m_tiles);
 }
 
 /* Row-major W[N, K] (N % 32 == 0, K % 64 == 0) -> fragment order: the 16 bytes that lane l = 32 g + n % 32
  * feeds to slice j of K step ks of column block nb = n / 32, i.e. W[n][64 ks + 32 g + 8 j .. + 8], go to
  * 16-byte slot ((nb * K/64 + ks) * 4 + j) * 64 + l.  A block of 32 rows occupies the same 32 K elements
  * in both layouts. */
-__global__ void vt_frag_layout_kernel(u32x4 *out, const uint16_t *W, size_t n_slots, int K) {
+/* pair: W is a gate|up matrix with (gate, up) rows interleaved; fragment column n' of every 64 takes row
+ * 64 (n'/64) + 2 (n' % 32) + (n' % 64) / 32, so that a wave of the product (64 columns) holds the gates of 32
+ * h columns in its first column block and their ups in the second. */
+__global__ void vt_frag_layout_kernel(u32x4 *out, const uint16_t *W, size_t n_slots, int K, int pair) {
     const int ksteps = K / GM_BK;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_slots; i += (size_t)gridDim.x * blockDim.x) {
         const int l = (int)(i & 63), j = (int)((i >> 6) & 3);
         const size_t blk = i >> 8;
         const int ks = (int)(blk % ksteps);
         const size_t nb = blk / ksteps;
-        const size_t n = nb * 32 + (l & 31);
+        size_t n = nb * 32 + (l & 31);
+        if (pair) n = (nb >> 1) * 64 + 2 * (l & 31) + (nb & 1);
         out[i] = gm_ld(W + n * K + 64 * ks + 32 * (l >> 5) + 8 * j);
     }
 }
 
-void vt_launch_frag_layout(uint16_t *d_Wf, const uint16_t *d_W, int N, int K) {
+void vt_launch_frag_layout(uint16_t *d_Wf, const uint16_t *d_W, int N, int K, int pair) {
     const size_t n_slots = (size_t)N * K / 8;
     hipLaunchKernelGGL(vt_frag_layout_kernel, dim3(gm_blocks(n_slots)), dim3(256), 0, g_vt.stream, (u32x4 *)d_Wf, d_W,
-                       n_slots, K);
+                       n_slots, K, pair);
 }
 
 int vt_gemm_shape_ok(int M, int N, int K, int splits) {
@@ -593,6 +626,43 @@ void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, s
                             const float *d_tail, int tail_planes, size_t tail_stride) {
     hipLaunchKernelGGL(vt_swiglu_split_kernel, dim3(gm_blocks(n_out / 4)), dim3(256), 0, g_vt.stream, d_hi, d_lo,
                        d_gu, n_out / 4, tail_col0, d_tail, tail_planes, tail_stride);
+}
+
+/* The K-cut tail of the paired gate|up product: tail [planes][rows, tw] fp32 in the paired column order
+ * (of every 64 columns the first 32 are gates, the other 32 the ups of the same h columns) -> the
+ * (hi, lo) planes of SiLU(gate) * up at h columns h_col0 .. h_col0 + tw/2 (row pitch ldh).  A thread owns 4
+ * consecutive h columns. */
+__global__ void vt_swiglu_pair_tail_kernel(uint16_t *hi, uint16_t *lo, int ldh, int h_col0, const float *tail,
+                                           int planes, size_t stride, int rows, int tw) {
+    const int per_row = tw / 8;                                   /* threads per row */
+    const size_t total = (size_t)rows * per_row;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int row = (int)(i / per_row), q = (int)(i % per_row);
+        const int blk = q >> 3, c = (q & 7) * 4;
+        const float *tp = tail + (size_t)row * tw + 64 * blk + c;
+        f32x4 g = *reinterpret_cast<const f32x4 *>(tp), u = *reinterpret_cast<const f32x4 *>(tp + 32);
+        for (int p = 1; p < planes; p++) {
+            const f32x4 g2 = *reinterpret_cast<const f32x4 *>(tp + p * stride);
+            const f32x4 u2 = *reinterpret_cast<const f32x4 *>(tp + p * stride + 32);
+            g.x = __fadd_rn(g.x, g2.x); g.y = __fadd_rn(g.y, g2.y); g.z = __fadd_rn(g.z, g2.z); g.w = __fadd_rn(g.w, g2.w);
+            u.x = __fadd_rn(u.x, u2.x); u.y = __fadd_rn(u.y, u2.y); u.z = __fadd_rn(u.z, u2.z); u.w = __fadd_rn(u.w, u2.w);
+        }
+        const float a = __fmul_rn(__fdiv_rn(g.x, __fadd_rn(1.0f, expf(-g.x))), u.x);
+        const float b = __fmul_rn(__fdiv_rn(g.y, __fadd_rn(1.0f, expf(-g.y))), u.y);
+        const float cc = __fmul_rn(__fdiv_rn(g.z, __fadd_rn(1.0f, expf(-g.z))), u.z);
+        const float d = __fmul_rn(__fdiv_rn(g.w, __fadd_rn(1.0f, expf(-g.w))), u.w);
+        u32x2 sph, spl;
+        vt_split_planes4(a, b, cc, d, sph, spl);
+        const size_t at = (size_t)row * ldh + h_col0 + 32 * blk + c;
+        *reinterpret_cast<u32x2 *>(hi + at) = sph;
+        *reinterpret_cast<u32x2 *>(lo + at) = spl;
+    }
+}
+
+void vt_launch_swiglu_pair_tail(uint16_t *d_hi, uint16_t *d_lo, int ldh, int h_col0, const float *d_tail, int planes,
+                                size_t stride, int rows, int tw) {
+    hipLaunchKernelGGL(vt_swiglu_pair_tail_kernel, dim3(gm_blocks((size_t)rows * tw / 8)), dim3(256), 0, g_vt.stream,
+                       d_hi, d_lo, ldh, h_col0, d_tail, planes, stride, rows, tw);
 }
 
 /* C = sum of `splits` partial planes (fixed order), for callers that want the plain product. */

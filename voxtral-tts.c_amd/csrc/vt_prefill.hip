@@ -328,16 +328,18 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         if (frag) vt_launch_gemm_frag(part, VT_DIM, ps, hi, lo, F->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
         else vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
         vt_launch_residual_norm_split(x, part, sp_wo, ps, L->ffn_norm, hi, lo, seq_len);
+        /* with the fragment copies the SiLU(gate) * up planes come out of the product itself, into the wide
+         * area (free between q|k|v and the next layer), which the down projection then reads */
+        uint16_t *h_hi = (uint16_t *)wide, *h_lo = h_hi + n_plane;
         if (frag && m_tiles != 4) {
-            vt_launch_gemm_frag(wide, 2 * VT_FFN, 0, hi, lo, F->w13, seq_len, 2 * VT_FFN, VT_DIM, 1);
-            vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, 0, NULL, 0, 0);
+            vt_launch_gemm_frag_swiglu(h_hi, h_lo, VT_FFN, NULL, hi, lo, F->w13, seq_len, 2 * VT_FFN, 0, VT_DIM, 1);
         } else if (frag) {
             /* 4 M tiles x 72 N tiles of 256 columns are 288 items for 256 CUs: the last 8 N tiles get their K cut
              * in VT_W13_TAIL_CUT and every workgroup takes one of those cuts after its whole tile, in the same
              * launch, instead of 32 workgroups running a second round alone */
             const int tail = 8 * 256, main_cols = 2 * VT_FFN - tail;
-            vt_launch_gemm_frag_tail(wide, 2 * VT_FFN, part, hi, lo, F->w13, seq_len, main_cols, tail, VT_DIM, VT_W13_TAIL_CUT);
-            vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, main_cols, part, VT_W13_TAIL_CUT, S * tail);
+            vt_launch_gemm_frag_swiglu(h_hi, h_lo, VT_FFN, part, hi, lo, F->w13, seq_len, main_cols, tail, VT_DIM, VT_W13_TAIL_CUT);
+            vt_launch_swiglu_pair_tail(h_hi, h_lo, VT_FFN, main_cols / 2, part, VT_W13_TAIL_CUT, S * tail, seq_len, tail);
         } else if (tail_cols) {
             /* 4 M tiles x 144 N tiles are 576 workgroups for 512 slots: the last 16 N tiles get their
              * K cut in 4 instead of running as a nearly empty second round */
@@ -350,7 +352,7 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
             vt_launch_gemm(wide, hi, lo, L->w13, seq_len, 2 * VT_FFN, VT_DIM, 1);
             vt_launch_swiglu_split(hi, lo, wide, S * VT_FFN, 0, NULL, 0, 0);
         }
-        if (frag) vt_launch_gemm_frag(part, VT_DIM, ps, hi, lo, F->w2, seq_len, VT_DIM, VT_FFN, sp_w2);
+        if (frag) vt_launch_gemm_frag(part, VT_DIM, ps, h_hi, h_lo, F->w2, seq_len, VT_DIM, VT_FFN, sp_w2);
         else vt_launch_gemm(part, hi, lo, L->w2, seq_len, VT_DIM, VT_FFN, sp_w2);
         const float *next_norm = l + 1 < g_vt.n_dec_layers ? g_vt.h_layers[l + 1].attn_norm : NULL;
         vt_launch_residual_norm_split(x, part, sp_w2, ps, next_norm, hi, lo, seq_len);
@@ -402,8 +404,9 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
         const bool frag = F->wqkv && F->wo && F->w13 && F->w2;
         if (which == 2 && frag) {                       /* as in the prefill: main part + K-cut tail */
             const int tail = 8 * 256, main_cols = 2 * VT_FFN - tail;
-            vt_launch_gemm_frag_tail(out, 2 * VT_FFN, out + (size_t)S * 2 * VT_FFN, hi, lo, Wf[2], S, main_cols, tail, VT_DIM,
-                                     VT_W13_TAIL_CUT);
+            uint16_t *h_hi = (uint16_t *)out, *h_lo = h_hi + n_plane;
+            vt_launch_gemm_frag_swiglu(h_hi, h_lo, VT_FFN, out + (size_t)S * 2 * VT_FFN, hi, lo, Wf[2], S, main_cols, tail, VT_DIM,
+                                       VT_W13_TAIL_CUT);
         } else if (which == 2) {
             const int tail = 16 * 128, main_cols = 2 * VT_FFN - tail;
             vt_launch_gemm_ex(out, 2 * VT_FFN, 0, hi, lo, W[2], S, main_cols, VT_DIM, 1);
