@@ -182,7 +182,10 @@ def test_causal_attention_prefill_with_offset(hip, orc):
                                              S.KV_HEADS, S.HEAD_DIM, SCALE)
     hip.lib.tts_hip_sync()
     ref = orc.causal_attention(Q, K, V, seq, start + seq, start)
-    ok, mr, ma, bad = S.compare_tensors(ref, dO.to_numpy(np.float32, Q.shape), 1e-3, 1e-5)
+    # the sequence kernel feeds (hi, lo) bf16 pairs to the matrix cores (16 mantissa bits per operand):
+    # the reference's rule with the absolute floor scaled to the output, as for the seq > 1 linear
+    ok, mr, ma, bad = S.compare_tensors(ref, dO.to_numpy(np.float32, Q.shape), 1e-3,
+                                        1e-3 * float(np.sqrt(np.mean(ref.astype(np.float64) ** 2))))
     assert ok, (mr, ma, bad)
 
 

@@ -1,6 +1,6 @@
 """Sequence-level (prefill) kernels on the matrix cores against the oracle:
-the bf16 product on (hi, lo) activation planes, the causal attention on fp32
-MFMA tiles and the whole prefill at sequence length 512, through the C ABI.
+the bf16 product on (hi, lo) activation planes, the causal attention (both of its
+products on the same planes) and the whole prefill at sequence length 512, through the C ABI.
 The oracle's seq_len > 1 linear is the reference's triple loop
 (voxtral_tts_kernels.c:127-138); the bound is the path's 1e-3 per output
 vector, and a much tighter one (5e-5 of the row's rms: the sequential fp32 sum of
@@ -91,9 +91,15 @@ def test_causal_attention_tiles(hip, orc, seq, start):
     hip.check()
     ref = orc.causal_attention(Q, K, V, seq, start + seq, start)
     got = dO.to_numpy(np.float32, Q.shape)
-    ok, mr, ma, bad = S.compare_tensors(ref, got, 1e-3, 1e-5)
+    # Q, K, V and the probabilities enter the matrix cores as (hi, lo) bf16 pairs: 16 mantissa bits, an
+    # error of up to 2^-17 of each operand, i.e. absolute errors of a few 1e-5 on sums of O(1) terms that
+    # may cancel.  The reference's rule with its attention rtol (test_kernels.c:79-116, :463-468) and the
+    # absolute floor scaled to the output (1e-3 of its rms), then every row against its own rms.
+    ok, mr, ma, bad = S.compare_tensors(ref, got, 1e-3, 1e-3 * float(np.sqrt(np.mean(ref.astype(np.float64) ** 2))))
     assert ok, (mr, ma, bad)
-    rows_close(ref, got, f"attention {seq}+{start}", tight=1e-4)
+    # per row: the l2 error stays near 2^-17; the largest element error is 2^-16 of the largest term p v of
+    # its sum, which in a row of many keys is several times the row's rms (measured worst: 1.3e-4)
+    rows_close(ref, got, f"attention {seq}+{start}", tight=3e-4)
     for b in (dQ, dK, dV, dO):
         b.free()
 
@@ -138,10 +144,12 @@ def test_attention_first_key_only_and_equal_keys(hip):
     hip.lib.tts_hip_sync()
     got = dO.to_numpy(np.float32, Q.shape).reshape(seq, S.HEADS, S.HEAD_DIM)
     Vh = V.reshape(seq, S.KV_HEADS, S.HEAD_DIM).astype(np.float64)
+    # V passes through the (hi, lo) split: 16 mantissa bits, at most 2^-17 of |v| off per row
+    atol = 2.0 ** -16 * float(np.abs(V).max())
     for h in (0, 5, 31):
-        assert np.allclose(got[0, h], Vh[0, h // 4], rtol=0, atol=1e-6)
+        assert np.allclose(got[0, h], Vh[0, h // 4], rtol=0, atol=atol)
         for i in (1, 31, 32, 39):
-            assert np.allclose(got[i, h], Vh[: i + 1, h // 4].mean(axis=0), rtol=0, atol=2e-6)
+            assert np.allclose(got[i, h], Vh[: i + 1, h // 4].mean(axis=0), rtol=0, atol=atol)
 
 
 def _prefill_case(n_layers, chunks, kv_max, check_rows):

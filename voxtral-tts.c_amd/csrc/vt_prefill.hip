@@ -57,29 +57,52 @@ __global__ void vt_split_qkv_rope_kernel(const float *qkv, int planes, size_t pl
  *
  * Workgroup = (KV head, HPW of its 4 query heads, block of 16 queries), HPW*NSPLIT
  * waves: wave = (query head, key-tile residue).  The waves of one residue share 32-key
- * K and V tiles in LDS.  Scores are computed transposed, S^T = K Q^T, with
- * v_mfma_f32_16x16x4_f32, so that a lane owns one query: lane l holds query l%16 and
- * the keys 4*(l/16) + v of each 16-key block in accumulator element v.  The softmax
- * state is then per lane (two exchanges across the four lane groups per tile), and the
- * probabilities are already in the operand layout of the second product
- * O^T = V^T P^T, whose reduction index runs over the keys in that same order.
- * fp32 operands throughout.  Residues are merged through LDS at the end.
+ * K and V tiles in LDS, converted to (hi, lo) planes once, by the threads that fetched them, and
+ * laid out as the matrix instructions want them: K as [key][dim] (a lane's operand is 8 consecutive
+ * dims of a key), V transposed as [dim][lane group][8 key slots] (a lane's operand is the 8 keys of
+ * its group for one dim).  Both products run on the bf16 matrix cores
+ * (v_mfma_f32_16x16x32_bf16) with every fp32 operand split in (hi, lo) bf16 planes as in
+ * the projections: a b = hi_a hi_b + hi_a lo_b + lo_a hi_b, 16 mantissa bits per operand,
+ * fp32 accumulation; three such instructions take 3/16 of the time of the fp32 ones they
+ * replace.  Scores are computed transposed, S^T = K Q^T, so that a lane owns one query:
+ * lane l holds query l%16 and the keys 4*(l/16) + v of each 16-key block in accumulator
+ * element v.  The softmax state is then per lane (two exchanges across the four lane
+ * groups per tile), and the eight probabilities a lane holds are exactly its share of the
+ * reduction index of the second product O^T = V^T P^T (the k order inside a matrix
+ * instruction is free as long as both operands agree: slot j of lane group g stands for
+ * key 16*(j/4) + 4*g + j%4).  Residues are merged through LDS at the end.
  * 16-query blocks give 32 blocks per KV head at 512 queries: with HPW = 2 that is 512
  * workgroups whose work grows with the block index (causal), enough to keep 256 CUs
  * busy when long and short blocks follow each other. */
 #define PA_QT 16                  /* queries per workgroup */
-#define PA_KP 132                 /* tile pitch in floats: 16-byte reads over 16 keys cover all banks,
-                                     and rows 4 apart (the lane groups of the P V operand) do not collide */
-#define PA_TILE_FLOATS (2 * 32 * PA_KP)
+#define PA_KROW 272               /* bytes per key of a K plane: 128 bf16 + 16 (16-byte reads over 16 keys cover all banks) */
+#define PA_VROW 80                /* bytes per dim of a V plane: 4 lane groups x 8 key slots + 16 */
+#define PA_KPLANE (32 * PA_KROW)
+#define PA_VPLANE (VT_HEAD_DIM * PA_VROW)
+#define PA_TILE_BYTES (2 * PA_KPLANE + 2 * PA_VPLANE)
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+/* eight consecutive k of a matrix-core operand from two fp32 quads: (hi, lo) planes */
+__device__ __forceinline__ void pa_planes8(const f32x4 &a, const f32x4 &b, bf16x8 &hi, bf16x8 &lo) {
+    unsigned h0, h1, h2, h3, l0, l1, l2, l3;
+    vt_split_planes2(a.x, a.y, h0, l0);
+    vt_split_planes2(a.z, a.w, h1, l1);
+    vt_split_planes2(b.x, b.y, h2, l2);
+    vt_split_planes2(b.z, b.w, h3, l3);
+    hi = __builtin_bit_cast(bf16x8, u32x4{h0, h1, h2, h3});
+    lo = __builtin_bit_cast(bf16x8, u32x4{l0, l1, l2, l3});
+}
 
 template <int NSPLIT, int HPW>
 __global__ void __launch_bounds__(64 * HPW * NSPLIT)
 vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, const float *Q,
                             int q_stride, const float *Kc, const float *Vc, int S,
                             int start_pos, float scale) {
-    extern __shared__ __attribute__((aligned(16))) float pa_lds[];
+    extern __shared__ __attribute__((aligned(16))) unsigned char pa_lds[];
     constexpr int GT = 64 * HPW;                         /* threads of a residue group */
     constexpr int NLD = 1024 / GT;                       /* 16-byte loads per thread and tile */
+    static_assert(GT == 128, "a staging thread owns the 8 key slots of one lane group");
     const int kvh = (int)blockIdx.x / (4 / HPW), hsub = (int)blockIdx.x % (4 / HPW);
     /* long blocks first: the last query block has the most keys */
     const int qt = (int)gridDim.y - 1 - (int)blockIdx.y;
@@ -90,16 +113,34 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
     const int q0 = qt * PA_QT;
     const int my_q = q0 + li;
     const int head = kvh * 4 + hsub * HPW + hq;
-    float *Kt = pa_lds + (size_t)pz * PA_TILE_FLOATS, *Vt = Kt + 32 * PA_KP;
+    unsigned char *Kt = pa_lds + (size_t)pz * PA_TILE_BYTES, *Vt = Kt + 2 * PA_KPLANE;   /* hi plane, then lo */
 
-    /* this lane's query: dims 32*g .. 32*g+31 */
-    float qreg[32];
+    /* The workgroups of one blockIdx.x run on one XCD and walk the same K and V rows, tile by tile, at the
+     * same pace: left alone, every tile is a miss in that XCD's L2 for all of them at the moment they need
+     * it, and each step pays the full memory latency.  So they first touch all the rows between them, one
+     * 128-byte line per lane and request (K and V rows are 4 lines each), which starts every line on its way
+     * into the L2 at once.  The values are dropped at the end of the kernel. */
+    unsigned warm[4];
     {
-        const float *qp = Q + (size_t)(my_q < S ? my_q : S - 1) * q_stride + head * VT_HEAD_DIM + 32 * g;
+        const int n_lines = (start_pos + S) * 8, stride = (int)(gridDim.y * blockDim.x);
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const f32x4 v = reinterpret_cast<const f32x4 *>(qp)[i];
-            qreg[4 * i] = v.x; qreg[4 * i + 1] = v.y; qreg[4 * i + 2] = v.z; qreg[4 * i + 3] = v.w;
+        for (int k = 0; k < 4; k++) {
+            int j = (int)blockIdx.y * (int)blockDim.x + t + k * stride;
+            j = j < n_lines ? j : n_lines - 1;
+            const int which = j & 1, row = j >> 3, line = (j >> 1) & 3;
+            warm[k] = *reinterpret_cast<const unsigned *>((which ? Vc : Kc) + (size_t)row * VT_KV_DIM + kvh * VT_HEAD_DIM + line * 32);
+        }
+    }
+
+    /* this lane's query as the B operand of K Q^T: dims 8*g + 32*ks .. + 8 for K step ks, both planes */
+    bf16x8 qhi[4], qlo[4];
+    {
+        const float *qp = Q + (size_t)(my_q < S ? my_q : S - 1) * q_stride + head * VT_HEAD_DIM + 8 * g;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const f32x4 a = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[0];
+            const f32x4 b = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[1];
+            pa_planes8(a, b, qhi[ks], qlo[ks]);
         }
     }
     f32x4 o[8];
@@ -112,16 +153,18 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
     const int nsteps = (ntiles + NSPLIT - 1) / NSPLIT;
     const int kv_rows = start_pos + S;
 
-    /* staging: the threads of a residue group move 32 rows x 512 B of K and of V */
+    /* staging: the threads of a residue group move 32 rows x 512 B of K and of V.  Thread (sg, cg) takes
+     * the 4 dims 4*cg .. of the 8 keys that lane group sg meets in the second product (slot j: key
+     * 16*(j/4) + 4*sg + j%4). */
+    const int sg = tl >> 5, cg = tl & 31;
     f32x4 rk[NLD], rv[NLD];
     auto fetch = [&](int tile) {
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            const int c = tl + GT * i, row = c >> 5, col = (c & 31) * 4;
-            int kr = tile * 32 + row;
+            int kr = tile * 32 + 16 * (i >> 2) + 4 * sg + (i & 3);
             if (kr >= kv_rows) kr = kv_rows - 1;
-            rk[i] = *reinterpret_cast<const f32x4 *>(Kc + (size_t)kr * VT_KV_DIM + kvh * VT_HEAD_DIM + col);
-            rv[i] = *reinterpret_cast<const f32x4 *>(Vc + (size_t)kr * VT_KV_DIM + kvh * VT_HEAD_DIM + col);
+            rk[i] = *reinterpret_cast<const f32x4 *>(Kc + (size_t)kr * VT_KV_DIM + kvh * VT_HEAD_DIM + 4 * cg);
+            rv[i] = *reinterpret_cast<const f32x4 *>(Vc + (size_t)kr * VT_KV_DIM + kvh * VT_HEAD_DIM + 4 * cg);
         }
     };
     /* Every request of the loop below is unconditional (a tile index beyond the last visible one
@@ -137,9 +180,18 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
         if (valid) {
 #pragma unroll
             for (int i = 0; i < NLD; i++) {
-                const int c = tl + GT * i, row = c >> 5, col = (c & 31) * 4;
-                *reinterpret_cast<f32x4 *>(Kt + row * PA_KP + col) = rk[i];
-                *reinterpret_cast<f32x4 *>(Vt + row * PA_KP + col) = rv[i];
+                const int row = 16 * (i >> 2) + 4 * sg + (i & 3);
+                u32x2 h, l;
+                vt_split_planes4(rk[i].x, rk[i].y, rk[i].z, rk[i].w, h, l);
+                *reinterpret_cast<u32x2 *>(Kt + row * PA_KROW + 8 * cg) = h;
+                *reinterpret_cast<u32x2 *>(Kt + PA_KPLANE + row * PA_KROW + 8 * cg) = l;
+            }
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                bf16x8 h, l;
+                pa_planes8(f32x4{rv[0][d], rv[1][d], rv[2][d], rv[3][d]}, f32x4{rv[4][d], rv[5][d], rv[6][d], rv[7][d]}, h, l);
+                *reinterpret_cast<bf16x8 *>(Vt + (4 * cg + d) * PA_VROW + 16 * sg) = h;
+                *reinterpret_cast<bf16x8 *>(Vt + PA_VPLANE + (4 * cg + d) * PA_VROW + 16 * sg) = l;
             }
         }
         __syncthreads();
@@ -147,18 +199,19 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
         __builtin_amdgcn_sched_barrier(0);               /* requests first, products behind them */
         if (!valid) continue;
 
-        /* S^T = K Q^T: reduction step (j, e) pairs dim 32*g + 4*j + e of key and query */
+        /* S^T = K Q^T: K step ks pairs the dims 8*g + 32*ks .. + 8 of key 16*kb + li and of the query */
         f32x4 s[2];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
             s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const f32x4 kf = *reinterpret_cast<const f32x4 *>(Kt + (16 * kb + li) * PA_KP + 32 * g + 4 * j);
-                s[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.x, qreg[4 * j], s[kb], 0, 0, 0);
-                s[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.y, qreg[4 * j + 1], s[kb], 0, 0, 0);
-                s[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.z, qreg[4 * j + 2], s[kb], 0, 0, 0);
-                s[kb] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf.w, qreg[4 * j + 3], s[kb], 0, 0, 0);
+            for (int ks = 0; ks < 4; ks++) {
+                const unsigned char *kp = Kt + (16 * kb + li) * PA_KROW + 16 * g + 64 * ks;
+                const bf16x8 khi = *reinterpret_cast<const bf16x8 *>(kp);
+                const bf16x8 klo = *reinterpret_cast<const bf16x8 *>(kp + PA_KPLANE);
+                s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(klo, qhi[ks], s[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(khi, qlo[ks], s[kb], 0, 0, 0);
+                s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(khi, qhi[ks], s[kb], 0, 0, 0);
             }
         }
         /* online softmax for this lane's query; element v of block kb is key 16*kb + 4*g + v */
@@ -188,22 +241,25 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
         m = mn;
 #pragma unroll
         for (int b = 0; b < 8; b++) o[b] = o[b] * corr;
-        /* O^T += V^T P^T: reduction step (kb, v) pairs key 16*kb + 4*g + v with s[kb][v] */
+        /* O^T += V^T P^T: slot j of this lane group is key 16*(j/4) + 4*g + j%4, whose probability is
+         * s[j/4][j%4]; the A operand of dim block b is that key's column 16*b + li of V */
+        bf16x8 phi, plo;
+        pa_planes8(s[0], s[1], phi, plo);
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const float *vrow = Vt + (16 * kb + 4 * g + v) * PA_KP + li;
-#pragma unroll
-                for (int b = 0; b < 8; b++)
-                    o[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(vrow[16 * b], s[kb][v], o[b], 0, 0, 0);
-            }
+        for (int b = 0; b < 8; b++) {
+            const unsigned char *vp = Vt + (16 * b + li) * PA_VROW + 16 * g;
+            const bf16x8 vhi = *reinterpret_cast<const bf16x8 *>(vp);
+            const bf16x8 vlo = *reinterpret_cast<const bf16x8 *>(vp + PA_VPLANE);
+            o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vlo, phi, o[b], 0, 0, 0);
+            o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vhi, plo, o[b], 0, 0, 0);
+            o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vhi, phi, o[b], 0, 0, 0);
+        }
     }
 
     /* merge the residues: residue r > 0 parks (m, l, O) in LDS, residue 0 folds them in */
     if (NSPLIT > 1) {
         __syncthreads();
-        float *park = pa_lds;                            /* [NSPLIT-1][HPW][34][64 lanes] */
+        float *park = reinterpret_cast<float *>(pa_lds);  /* [NSPLIT-1][HPW][34][64 lanes] */
         for (int r = 1; r < NSPLIT; r++) {
             float *slot = park + ((size_t)((r - 1) * HPW + hq) * 34) * 64 + lane;
             if (pz == r) {
@@ -229,6 +285,7 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
             __syncthreads();
         }
     }
+    asm volatile("" ::"v"(warm[0]), "v"(warm[1]), "v"(warm[2]), "v"(warm[3]));
     if (pz != 0 || my_q >= S) return;
     float L = lsum + __shfl_xor(lsum, 16);
     L += __shfl_xor(L, 32);
@@ -253,11 +310,13 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
     }
 }
 
+#ifndef PA_NSPLIT
 #define PA_NSPLIT 2
+#endif
 #define PA_HPW 2
 
 static size_t pa_lds_bytes(void) {
-    size_t tiles = sizeof(float) * (size_t)PA_NSPLIT * PA_TILE_FLOATS;
+    size_t tiles = (size_t)PA_NSPLIT * PA_TILE_BYTES;
     size_t park = sizeof(float) * (size_t)(PA_NSPLIT - 1) * PA_HPW * 34 * 64;
     return tiles > park ? tiles : park;
 }
