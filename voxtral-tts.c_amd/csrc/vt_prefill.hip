@@ -18,15 +18,16 @@
 /* ---- RoPE + cache append ------------------------------------------------------- */
 
 /* qkv [S,6144] (the sum of `planes` split-K planes, `plane_stride` floats apart) ->
- * q [S,4096] with RoPE, cache rows start_pos.. (k with RoPE, v) */
+ * q [S,4096] with RoPE, cache rows start_pos.. (k with RoPE, v); only the columns from col0 on (a
+ * multiple of 4; VT_Q_DIM: the cache rows alone, for an attention that takes q from the planes itself) */
 __global__ void vt_split_qkv_rope_kernel(const float *qkv, int planes, size_t plane_stride, float *q,
-                                         float *kc, float *vc, const float *rope, int start_pos, int S) {
+                                         float *kc, float *vc, const float *rope, int start_pos, int S, int col0) {
     /* a thread owns two adjacent RoPE pairs: 16-byte loads and stores */
-    const int quads = VT_QKV_DIM / 4;
+    const int quads = (VT_QKV_DIM - col0) / 4;
     const size_t total = (size_t)S * quads;
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (size_t)gridDim.x * blockDim.x) {
-        const int s = (int)(i / quads), g = (int)(i % quads) * 4;
+        const int s = (int)(i / quads), g = col0 + (int)(i % quads) * 4;
         f32x4 ab = *reinterpret_cast<const f32x4 *>(qkv + (size_t)s * VT_QKV_DIM + g);
         for (int p = 1; p < planes; p++) {
             const f32x4 w = *reinterpret_cast<const f32x4 *>(qkv + p * plane_stride + (size_t)s * VT_QKV_DIM + g);
@@ -97,8 +98,8 @@ __device__ __forceinline__ void pa_planes8(const f32x4 &a, const f32x4 &b, bf16x
 template <int NSPLIT, int HPW>
 __global__ void __launch_bounds__(64 * HPW * NSPLIT)
 vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, const float *Q,
-                            int q_stride, const float *Kc, const float *Vc, int S,
-                            int start_pos, float scale) {
+                            int q_stride, int q_planes, size_t q_plane_stride, const float *rope,
+                            const float *Kc, const float *Vc, int S, int start_pos, float scale) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pa_lds[];
     constexpr int GT = 64 * HPW;                         /* threads of a residue group */
     constexpr int NLD = 1024 / GT;                       /* 16-byte loads per thread and tile */
@@ -135,11 +136,31 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
     /* this lane's query as the B operand of K Q^T: dims 8*g + 32*ks .. + 8 for K step ks, both planes */
     bf16x8 qhi[4], qlo[4];
     {
-        const float *qp = Q + (size_t)(my_q < S ? my_q : S - 1) * q_stride + head * VT_HEAD_DIM + 8 * g;
+        /* Q as it is, or (rope != NULL) the raw product: the sum of q_planes split-K planes, rotated here
+         * (adjacent pairs, voxtral_tts_kernels.c:616-634; the table holds (cos, sin) per pair) */
+        const int qrow = my_q < S ? my_q : S - 1;
+        const float *qp = Q + (size_t)qrow * q_stride + head * VT_HEAD_DIM + 8 * g;
+        const float *cs = rope ? rope + (size_t)(start_pos + qrow) * VT_HEAD_DIM + 8 * g : NULL;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            const f32x4 a = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[0];
-            const f32x4 b = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[1];
+            f32x4 a = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[0];
+            f32x4 b = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[1];
+            if (rope) {
+                for (int p = 1; p < q_planes; p++) {
+                    const f32x4 a2 = reinterpret_cast<const f32x4 *>(qp + p * q_plane_stride + 32 * ks)[0];
+                    const f32x4 b2 = reinterpret_cast<const f32x4 *>(qp + p * q_plane_stride + 32 * ks)[1];
+                    a.x = __fadd_rn(a.x, a2.x); a.y = __fadd_rn(a.y, a2.y); a.z = __fadd_rn(a.z, a2.z); a.w = __fadd_rn(a.w, a2.w);
+                    b.x = __fadd_rn(b.x, b2.x); b.y = __fadd_rn(b.y, b2.y); b.z = __fadd_rn(b.z, b2.z); b.w = __fadd_rn(b.w, b2.w);
+                }
+                const f32x4 c0 = reinterpret_cast<const f32x4 *>(cs + 32 * ks)[0];
+                const f32x4 c1 = reinterpret_cast<const f32x4 *>(cs + 32 * ks)[1];
+                const f32x4 ra = {__fsub_rn(__fmul_rn(a.x, c0.x), __fmul_rn(a.y, c0.y)), __fadd_rn(__fmul_rn(a.x, c0.y), __fmul_rn(a.y, c0.x)),
+                                  __fsub_rn(__fmul_rn(a.z, c0.z), __fmul_rn(a.w, c0.w)), __fadd_rn(__fmul_rn(a.z, c0.w), __fmul_rn(a.w, c0.z))};
+                const f32x4 rb = {__fsub_rn(__fmul_rn(b.x, c1.x), __fmul_rn(b.y, c1.y)), __fadd_rn(__fmul_rn(b.x, c1.y), __fmul_rn(b.y, c1.x)),
+                                  __fsub_rn(__fmul_rn(b.z, c1.z), __fmul_rn(b.w, c1.w)), __fadd_rn(__fmul_rn(b.z, c1.w), __fmul_rn(b.w, c1.z))};
+                a = ra;
+                b = rb;
+            }
             pa_planes8(a, b, qhi[ks], qlo[ks]);
         }
     }
@@ -321,10 +342,12 @@ static size_t pa_lds_bytes(void) {
     return tiles > park ? tiles : park;
 }
 
-/* Q rows are q_stride floats apart; out / (out_hi, out_lo) are [S,4096], each optional. */
-void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
-                                 int q_stride, const float *d_K, const float *d_V, int S, int start_pos,
-                                 float scale) {
+/* Q rows are q_stride floats apart; out / (out_hi, out_lo) are [S,4096], each optional.  d_rope != NULL: d_Q
+ * holds q_planes split-K planes (q_plane_stride floats apart) of the raw q product, to be summed and
+ * rotated with the table rows start_pos .. by the kernel. */
+void vt_launch_prefill_attention_raw(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
+                                     int q_stride, int q_planes, size_t q_plane_stride, const float *d_rope,
+                                     const float *d_K, const float *d_V, int S, int start_pos, float scale) {
     static int attr_set = 0;
     if (!attr_set) {
         if (vt_check(hipFuncSetAttribute((const void *)vt_prefill_attention_kernel<PA_NSPLIT, PA_HPW>,
@@ -335,8 +358,14 @@ void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, c
     }
     hipLaunchKernelGGL((vt_prefill_attention_kernel<PA_NSPLIT, PA_HPW>),
                        dim3(VT_KV_HEADS * (4 / PA_HPW), (S + PA_QT - 1) / PA_QT), dim3(64 * PA_HPW * PA_NSPLIT),
-                       pa_lds_bytes(), g_vt.stream, d_out, d_hi, d_lo, d_Q, q_stride, d_K, d_V, S, start_pos,
-                       scale);
+                       pa_lds_bytes(), g_vt.stream, d_out, d_hi, d_lo, d_Q, q_stride, q_planes, q_plane_stride, d_rope,
+                       d_K, d_V, S, start_pos, scale);
+}
+
+void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
+                                 int q_stride, const float *d_K, const float *d_V, int S, int start_pos,
+                                 float scale) {
+    vt_launch_prefill_attention_raw(d_out, d_hi, d_lo, d_Q, q_stride, 1, 0, NULL, d_K, d_V, S, start_pos, scale);
 }
 
 /* ---- backbone prefill ------------------------------------------------------------ */
@@ -381,9 +410,11 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         const bool frag = F->wqkv && F->wo && F->w13 && F->w2;
         if (frag) vt_launch_gemm_frag(wide, VT_QKV_DIM, S * VT_QKV_DIM, hi, lo, F->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
         else vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
-        hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(ew_blocks(S * VT_QKV_DIM / 4)), dim3(256), 0, st,
-                           wide, sp_qkv, S * VT_QKV_DIM, q, kc, vc, g_vt.d_rope, start_pos, seq_len);
-        vt_launch_prefill_attention(NULL, hi, lo, q, VT_Q_DIM, kc, vc, seq_len, start_pos, VT_ATT_SCALE);
+        /* k (rotated) and v into the cache; the attention takes q from the product's planes itself */
+        hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(ew_blocks(S * 2 * VT_KV_DIM / 4)), dim3(256), 0, st,
+                           wide, sp_qkv, S * VT_QKV_DIM, q, kc, vc, g_vt.d_rope, start_pos, seq_len, VT_Q_DIM);
+        vt_launch_prefill_attention_raw(NULL, hi, lo, wide, VT_QKV_DIM, sp_qkv, S * VT_QKV_DIM, g_vt.d_rope, kc, vc,
+                                        seq_len, start_pos, VT_ATT_SCALE);
         if (frag) vt_launch_gemm_frag(part, VT_DIM, ps, hi, lo, F->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
         else vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
         vt_launch_residual_norm_split(x, part, sp_wo, ps, L->ffn_norm, hi, lo, seq_len);
