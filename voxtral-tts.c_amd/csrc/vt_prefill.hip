@@ -78,8 +78,14 @@ __global__ void vt_split_qkv_rope_kernel(const float *qkv, int planes, size_t pl
 #define PA_QT 16                  /* queries per workgroup */
 #define PA_KROW 272               /* bytes per key of a K plane: 128 bf16 + 16 (16-byte reads over 16 keys cover all banks) */
 #define PA_VROW 80                /* bytes per dim of a V plane: 4 lane groups x 8 key slots + 16 */
+/* Dim d of V sits in row (d % 4) * 34 + d / 4 of its plane: a staging thread writes the same key slots of 4
+ * consecutive dims, and a wave of them dims 4 apart, which in dim order would be rows 320 bytes apart, two
+ * bank groups for eight lanes.  This way the lanes of a 16-byte write are consecutive rows, and the eight
+ * lanes of a 16-byte read (dims li = 0 .. 7 of a block: rows (li % 4) * 34 + li / 4) still cover all banks,
+ * because 34 * 80 bytes is 2 of the 8 bank groups further on. */
+#define PA_VSKEW 34
 #define PA_KPLANE (32 * PA_KROW)
-#define PA_VPLANE (VT_HEAD_DIM * PA_VROW)
+#define PA_VPLANE ((3 * PA_VSKEW + VT_HEAD_DIM / 4) * PA_VROW)
 #define PA_TILE_BYTES (2 * PA_KPLANE + 2 * PA_VPLANE)
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -105,8 +111,12 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
     constexpr int NLD = 1024 / GT;                       /* 16-byte loads per thread and tile */
     static_assert(GT == 128, "a staging thread owns the 8 key slots of one lane group");
     const int kvh = (int)blockIdx.x / (4 / HPW), hsub = (int)blockIdx.x % (4 / HPW);
-    /* long blocks first: the last query block has the most keys */
-    const int qt = (int)gridDim.y - 1 - (int)blockIdx.y;
+    /* The last query block has the most keys.  Workgroups are handed to the CUs in launch order, one per
+     * CU and then a second one each: the first half of the launch takes the long blocks in descending
+     * order, the second half the short ones in ascending order, so that every CU gets a long block and
+     * the short one that makes up the same total. */
+    const int ny = (int)gridDim.y, half = (ny + 1) / 2;
+    const int qt = (int)blockIdx.y < half ? ny - 1 - (int)blockIdx.y : (int)blockIdx.y - half;
     const int t = (int)threadIdx.x, lane = t & 63, wave = t >> 6;
     const int hq = wave % HPW, pz = wave / HPW;
     const int tl = hq * 64 + lane;                       /* thread index inside the residue group */
@@ -179,13 +189,22 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
      * 16*(j/4) + 4*sg + j%4). */
     const int sg = tl >> 5, cg = tl & 31;
     f32x4 rk[NLD], rv[NLD];
+    /* buffer loads: the tile's first row as the scalar offset, this thread's row and columns as a vector
+     * offset that never changes (no 64-bit address arithmetic per load), and rows past the end of the
+     * cache read as zeros (their keys are masked) */
+    const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc((void *)(Kc + kvh * VT_HEAD_DIM), 0,
+                                                                          kv_rows * VT_KV_DIM * 4 - kvh * VT_HEAD_DIM * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc((void *)(Vc + kvh * VT_HEAD_DIM), 0,
+                                                                          kv_rows * VT_KV_DIM * 4 - kvh * VT_HEAD_DIM * 4, 0x00020000);
+    int voff[NLD];
+#pragma unroll
+    for (int i = 0; i < NLD; i++) voff[i] = (16 * (i >> 2) + 4 * sg + (i & 3)) * (VT_KV_DIM * 4) + 16 * cg;
     auto fetch = [&](int tile) {
+        const int soff = __builtin_amdgcn_readfirstlane(tile) * (32 * VT_KV_DIM * 4);
 #pragma unroll
         for (int i = 0; i < NLD; i++) {
-            int kr = tile * 32 + 16 * (i >> 2) + 4 * sg + (i & 3);
-            if (kr >= kv_rows) kr = kv_rows - 1;
-            rk[i] = *reinterpret_cast<const f32x4 *>(Kc + (size_t)kr * VT_KV_DIM + kvh * VT_HEAD_DIM + 4 * cg);
-            rv[i] = *reinterpret_cast<const f32x4 *>(Vc + (size_t)kr * VT_KV_DIM + kvh * VT_HEAD_DIM + 4 * cg);
+            rk[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(k_rs, voff[i], soff, 0));
+            rv[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(v_rs, voff[i], soff, 0));
         }
     };
     /* Every request of the loop below is unconditional (a tile index beyond the last visible one
@@ -211,8 +230,8 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
             for (int d = 0; d < 4; d++) {
                 bf16x8 h, l;
                 pa_planes8(f32x4{rv[0][d], rv[1][d], rv[2][d], rv[3][d]}, f32x4{rv[4][d], rv[5][d], rv[6][d], rv[7][d]}, h, l);
-                *reinterpret_cast<bf16x8 *>(Vt + (4 * cg + d) * PA_VROW + 16 * sg) = h;
-                *reinterpret_cast<bf16x8 *>(Vt + PA_VPLANE + (4 * cg + d) * PA_VROW + 16 * sg) = l;
+                *reinterpret_cast<bf16x8 *>(Vt + (d * PA_VSKEW + cg) * PA_VROW + 16 * sg) = h;
+                *reinterpret_cast<bf16x8 *>(Vt + PA_VPLANE + (d * PA_VSKEW + cg) * PA_VROW + 16 * sg) = l;
             }
         }
         __syncthreads();
@@ -268,7 +287,7 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
         pa_planes8(s[0], s[1], phi, plo);
 #pragma unroll
         for (int b = 0; b < 8; b++) {
-            const unsigned char *vp = Vt + (16 * b + li) * PA_VROW + 16 * g;
+            const unsigned char *vp = Vt + ((li & 3) * PA_VSKEW + 4 * b + (li >> 2)) * PA_VROW + 16 * g;
             const bf16x8 vhi = *reinterpret_cast<const bf16x8 *>(vp);
             const bf16x8 vlo = *reinterpret_cast<const bf16x8 *>(vp + PA_VPLANE);
             o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vlo, phi, o[b], 0, 0, 0);
