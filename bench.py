@@ -281,7 +281,7 @@ def bench_prefill(args):
         "tokens_per_s": round(PREFILL_LEN / (ms_step * 1e-3), 1),
         "tflops": round((gemm_fl + attn_fl) / ms_step / 1e9, 1),
         "roofline": {
-            "kernel": "vt_gemm_mfma_kernel (the four projection launches of one layer at M = 512)",
+            "kernel": "vt_gemm_wide_kernel (the four projection launches of one layer at M = 512)",
             "bound": "mfma",
             "achieved": round(achieved, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
@@ -862,7 +862,7 @@ def other_workloads(hip, kv_max):
     ms_layer = sum(lib.tts_hip_bench_kernel(i, 26) for i in range(4))
     achieved = 2.0 * PREFILL_LEN * LAYER_WEIGHT_ELEMS / ms_layer / 1e9
     w["prefill, 512 tokens x 26 layers"] = {
-        "config": 3, "kernel": "vt_gemm_mfma_kernel (the projection launches of one layer)", "ms": round(ms, 3), "launches": 3,
+        "config": 3, "kernel": "vt_gemm_wide_kernel (the projection launches of one layer)", "ms": round(ms, 3), "launches": 3,
         "tokens_per_s": round(PREFILL_LEN / (ms * 1e-3), 1), "tflops_whole_prefill": round((gemm_fl + attn_fl) / ms / 1e9, 1),
         "us_products_per_layer": round(ms_layer * 1e3, 1), "achieved": round(achieved, 1), "unit": "TFLOP/s",
         "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "attention_us_per_layer": round(lib.tts_hip_bench_kernel(4, 26) * 1e3, 1)}
