@@ -176,7 +176,7 @@ struct vt_grid_sync {
  * of 256 workgroups are coherent loads served by the memory side, and spread over the copies
  * they do not queue on one channel. */
 #ifndef VT_FLAG_COPIES
-#define VT_FLAG_COPIES 8
+#define VT_FLAG_COPIES 4          /* 1 / 2 / 4 / 8 / 16 copies: 1.180 / 1.182 / 1.179 / 1.185 / 1.193 ms per launch (every copy is one more flag store per barrier) */
 #endif
 #define VT_FLAG_STRIDE 16384
 /* Words between the flags of two workgroups: partial writes to one 64-byte line are served one
@@ -184,7 +184,7 @@ struct vt_grid_sync {
  * a line see their stores acknowledged after 0.9 us, one flag to a line after 0.3 us), so the flags
  * are spread out; a poll then touches VT_FLAG_PAD times as many lines. */
 #ifndef VT_FLAG_PAD
-#define VT_FLAG_PAD 4
+#define VT_FLAG_PAD 8             /* with 4 copies, 4 / 6 / 8 / 12 / 16 words: 1.1805 / 1.179 / 1.1746 / 1.178 / 1.180 ms per launch */
 #endif
 #define VT_FLAG_LOADS 4           /* flags a lane polls: grids of up to 256 workgroups */
 #define VT_FLAG_ABORT_AT 8192     /* word of a copy that says "a workgroup has given up" (one word read by 256
