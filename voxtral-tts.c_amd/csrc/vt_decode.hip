@@ -116,18 +116,16 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
             return;
         vt_w13_body(ring, L, a, lds, [&] { vt_w2_prefetch(ring, L, VT_PART_HEAD); });
         if (!vt_barrier_then(gs, &s_flag, [&] { vt_w2_prefetch(ring, L, VT_PART_TAIL); }, tn)) return;
-        vt_w2_body(ring, L, a, lds, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1], VT_PART_HEAD); });
+        /* without a final norm the last layer's rows are the output: every workgroup writes its own and the
+         * kernel ends without a last hand-over (in place is fine: the input was last read two phases ago) */
+        const bool last_direct = !more && !a.final_norm;
+        vt_w2_body(ring, L, a, lds, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1], VT_PART_HEAD); }, last_direct);
+        if (last_direct) return;
         if (!vt_barrier_then(gs, &s_flag, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1], VT_PART_TAIL); }, tn))
             return;
         x_in = a.x;
     }
-    if (blockIdx.x == 0) {
-        if (a.final_norm) {
-            vt_block_rmsnorm<true>(a.out_hidden, a.x, a.final_norm, VT_DIM, VT_EPS, lds);
-        } else {
-            for (int i = (int)threadIdx.x; i < VT_DIM; i += (int)blockDim.x) a.out_hidden[i] = vt_ldc(a.x + i);
-        }
-    }
+    if (blockIdx.x == 0) vt_block_rmsnorm<true>(a.out_hidden, a.x, a.final_norm, VT_DIM, VT_EPS, lds);
 }
 
 /* ---- one kernel per phase ------------------------------------------------------ */

@@ -812,9 +812,12 @@ __device__ __forceinline__ void vt_w2_prefetch(u32x4 (&ring)[VT_RING], const vt_
     vt_ring_prefetch<9, 2>(ring, L.w2, VT_FFN, vt_w2_rows(), part);
 }
 
+/* out_direct: also write the result rows to a.out_hidden (the last layer of a step without a final norm:
+ * the output is then complete when the kernel ends and needs no hand-over of its own). */
 template <class AR = vt_nothing>
 __device__ __forceinline__ void vt_w2_body(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
-                                           const vt_step_args &a, float *lds, AR after_run = AR()) {
+                                           const vt_step_args &a, float *lds, AR after_run = AR(),
+                                           bool out_direct = false) {
     const vt_rows r = vt_w2_rows();
     float *lds_y = lds + VT_LDS_X;
     vt_stage(lds, a.h, VT_FFN);
@@ -827,7 +830,9 @@ __device__ __forceinline__ void vt_w2_body(u32x4 (&ring)[VT_RING], const vt_laye
     __syncthreads();
     for (int t = (int)threadIdx.x; t < r.wg_nrows; t += (int)blockDim.x) {
         const float y = lds_y[t] + lds_y[r.wg_nrows + t];
-        vt_stc(a.x + r.wg_row0 + t, (t == tr ? prev : vt_ldc(a.x + r.wg_row0 + t)) + y);
+        const float v = (t == tr ? prev : vt_ldc(a.x + r.wg_row0 + t)) + y;
+        vt_stc(a.x + r.wg_row0 + t, v);
+        if (out_direct) a.out_hidden[r.wg_row0 + t] = v;
     }
 }
 
