@@ -67,76 +67,66 @@ template <int PH> struct ac_shape {
 /* Activation rows are fetched into registers BEFORE the weight loads of a pass are
  * issued: a wave's loads return in order, so this way the planes can be built while
  * the weights are still streaming in. */
-struct ac_rows_regs { f32x4 v[AC_ROWS][2]; f32x4 g[2]; };
 struct ac_attn_regs { f32x4 q[3][4]; f32x4 kv[AC_ROWS * 2 * VT_KV_DIM / 4 / AC_THREADS]; };
 
-/* rows of 3072 = 768 groups of 4 columns: thread t owns group t, and group 512 + t when t < 256
- * (16-byte loads: half the load instructions of 8-byte ones for the same bytes) */
-__device__ __forceinline__ void ac_fetch_rows(ac_rows_regs &r, const float *src, int src_stride,
-                                              const float *gain) {
-    const int t = (int)threadIdx.x;
-    const bool two = t < 256;
+/* A wave's own K slice of the 6 rows.  The products of a wave read only the plane columns of its K slice
+ * (wave w: columns w * KW .. + KW), so a wave that fetches, scales and converts exactly those columns
+ * depends on no other wave before its first matrix instruction: no workgroup barrier between the rows'
+ * arrival and the products.  Behind an RMSNorm the planes then hold x * gain and the result is multiplied
+ * by 1/rms(x) in the epilogue, from the waves' partial sums of squares (red_ss[wave * 8 + m]). */
+template <int KW> struct ac_slice_regs {
+    static constexpr int NJ = (KW / 4 + 63) / 64;       /* 16-byte groups per lane and row */
+    f32x4 v[AC_ROWS][NJ];
+    f32x4 g[NJ];
+};
+
+template <int KW>
+__device__ __forceinline__ void ac_fetch_slice(ac_slice_regs<KW> &r, const float *src, int src_stride, const float *gain) {
+    constexpr int NJ = ac_slice_regs<KW>::NJ, G4 = KW / 4;
+    const int lane = vt_lane(), c0 = vt_wave() * KW;
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f}, one = {1.f, 1.f, 1.f, 1.f};
 #pragma unroll
     for (int m = 0; m < AC_ROWS; m++) {
-        const f32x4 *row = reinterpret_cast<const f32x4 *>(src + (size_t)m * src_stride);
-        r.v[m][0] = row[t];
-        r.v[m][1] = two ? row[512 + t] : zero;
+        const f32x4 *row = reinterpret_cast<const f32x4 *>(src + (size_t)m * src_stride + c0);
+#pragma unroll
+        for (int j = 0; j < NJ; j++) r.v[m][j] = (64 * (j + 1) <= G4 || lane + 64 * j < G4) ? row[lane + 64 * j] : zero;
     }
-    r.g[0] = one;
-    r.g[1] = one;
+#pragma unroll
+    for (int j = 0; j < NJ; j++) r.g[j] = one;
     if (gain) {
-        const f32x4 *g = reinterpret_cast<const f32x4 *>(gain);
-        r.g[0] = g[t];
-        r.g[1] = two ? g[512 + t] : one;
+        const f32x4 *g = reinterpret_cast<const f32x4 *>(gain + c0);
+#pragma unroll
+        for (int j = 0; j < NJ; j++) r.g[j] = (64 * (j + 1) <= G4 || lane + 64 * j < G4) ? g[lane + 64 * j] : one;
     }
 }
 
-/* registers -> (hi, lo) planes, optionally through RMSNorm */
-template <bool NORM>
-__device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned char *lo, int pitch,
-                                                  const ac_rows_regs &r, float *red) {
-    const int t = (int)threadIdx.x;
-    const bool two = t < 256;
-    float inv[AC_ROWS];
+template <bool NORM, int KW>
+__device__ __forceinline__ void ac_slice_to_planes(unsigned char *hi, unsigned char *lo, int pitch,
+                                                   const ac_slice_regs<KW> &r, float *red_ss) {
+    constexpr int NJ = ac_slice_regs<KW>::NJ, G4 = KW / 4;
+    const int lane = vt_lane(), c0 = vt_wave() * KW;
     if (NORM) {
 #pragma unroll
         for (int m = 0; m < AC_ROWS; m++) {
             float ss = 0.f;
 #pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const f32x4 v = r.v[m][j];                     /* zeros where this thread has no second group */
+            for (int j = 0; j < NJ; j++) {
+                const f32x4 v = r.v[m][j];
                 ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
             }
             ss = vt_wave_sum(ss);
-            if (vt_lane() == 0) red[vt_wave() * 8 + m] = ss;
+            if (lane == 0) red_ss[vt_wave() * 8 + m] = ss;
         }
-        __syncthreads();
-        /* lane m of every wave finishes row m (the division and the square root are some 50
-         * instructions; six of them in every lane were a third of this function), then the six
-         * values are broadcast from those lanes */
-        const int mrow = vt_lane() < AC_ROWS ? vt_lane() : 0;
-        float tot = 0.f;
-#pragma unroll
-        for (int w = 0; w < AC_WAVES; w++) tot += red[w * 8 + mrow];
-        const float mine = 1.0f / sqrtf(tot / (float)VT_DIM + VT_EPS);
-#pragma unroll
-        for (int m = 0; m < AC_ROWS; m++) inv[m] = vt_readlane(mine, m);
     }
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        if (j == 0 || two) {
-            const int c = 4 * (t + 512 * j);
+    for (int j = 0; j < NJ; j++) {
+        if (64 * (j + 1) <= G4 || lane + 64 * j < G4) {
+            const int c = c0 + 4 * (lane + 64 * j);
             const f32x4 g = r.g[j];
 #pragma unroll
             for (int m = 0; m < AC_ROWS; m++) {
                 f32x4 v = r.v[m][j];
-                if (NORM) {
-                    v.x = __fmul_rn(__fmul_rn(v.x, inv[m]), g.x);
-                    v.y = __fmul_rn(__fmul_rn(v.y, inv[m]), g.y);
-                    v.z = __fmul_rn(__fmul_rn(v.z, inv[m]), g.z);
-                    v.w = __fmul_rn(__fmul_rn(v.w, inv[m]), g.w);
-                }
+                if (NORM) { v.x = __fmul_rn(v.x, g.x); v.y = __fmul_rn(v.y, g.y); v.z = __fmul_rn(v.z, g.z); v.w = __fmul_rn(v.w, g.w); }
                 u32x2 sph, spl;
                 vt_split_planes4(v.x, v.y, v.z, v.w, sph, spl);
                 *reinterpret_cast<u32x2 *>(hi + m * pitch + 2 * c) = sph;
@@ -144,6 +134,9 @@ __device__ __forceinline__ void ac_rows_to_planes(unsigned char *hi, unsigned ch
             }
         }
     }
+    /* the wave's own stores before its own fragment reads: LDS serves a wave in order */
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 }
 
 /* Bidirectional attention over the 3 tokens of each branch, straight into the
@@ -258,9 +251,18 @@ __device__ __forceinline__ void ac_consume(const u32x4 (&wreg)[NL], const unsign
 }
 
 /* cross-wave sum of one unit and its epilogue; `red` is this unit's buffer */
+/* 1/rms of row m from the waves' partial sums of squares (wave-local planes) */
+__device__ __forceinline__ float ac_inv_rms_of(const float *red_ss, int m) {
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < AC_WAVES; w++) tot += red_ss[w * 8 + m];
+    return 1.0f / sqrtf(tot / (float)VT_DIM + VT_EPS);
+}
+
 template <int PH>
 __device__ __forceinline__ void ac_finish_unit(const ac_phase_args &a, float *red, int n0, f32x4 acc_hi,
-                                               f32x4 acc_lo, bool have_prev = false, float prev = 0.f) {
+                                               f32x4 acc_lo, bool have_prev = false, float prev = 0.f,
+                                               const float *red_ss = nullptr) {
     const int lane = vt_lane(), wave = vt_wave(), col = lane & 15, kg = lane >> 4;
     /* accumulator element v of lane l: activation row 4*(l/16) + v, weight row l%16 */
 #pragma unroll
@@ -279,6 +281,7 @@ __device__ __forceinline__ void ac_finish_unit(const ac_phase_args &a, float *re
                 g += red[(w * AC_ROWS + m) * 16 + 2 * j];
                 u += red[(w * AC_ROWS + m) * 16 + 2 * j + 1];
             }
+            if (red_ss) { const float inv = ac_inv_rms_of(red_ss, m); g = __fmul_rn(g, inv); u = __fmul_rn(u, inv); }
             a.out[(size_t)m * VT_FFN + (n0 >> 1) + j] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
         }
     } else if (t < AC_ROWS * 16 && (t & 15) < AC_RB) {
@@ -287,6 +290,7 @@ __device__ __forceinline__ void ac_finish_unit(const ac_phase_args &a, float *re
 #pragma unroll
         for (int w = 0; w < AC_WAVES; w++) y += red[(w * AC_ROWS + m) * 16 + n];
         if (PH == AC_QKV) {
+            if (red_ss) y = __fmul_rn(y, ac_inv_rms_of(red_ss, m));
             a.out[(size_t)m * VT_QKV_DIM + n0 + n] = y;
         } else {
             float *p = a.out + (size_t)m * VT_DIM + n0 + n;
@@ -329,18 +333,25 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
         prev = a.out[(size_t)(fin ? t >> 4 : 0) * VT_DIM + u * AC_RB + (fin ? t & 15 : 0)];
     }
 
+    /* behind an RMSNorm the planes hold x * gain; the epilogue multiplies by 1/rms(x) */
+    const float *scale_ss = (PH == AC_QKV || PH == AC_W13) ? red_ss : nullptr;
     if (SH::NPASS == 1) {
-        ac_rows_regs rr;
-        ac_attn_regs ra;
-        if (PH == AC_WO) ac_fetch_attn(ra, a.in); else ac_fetch_rows(rr, a.in, VT_DIM, a.gain);
-        ac_issue<PH>(w0, wbase + u * unit_stride);
-        if (PH == AC_WO) {
+        if (PH != AC_WO) {
+            /* every wave for itself: its K slice of the rows, no workgroup barrier before the products */
+            ac_slice_regs<SH::KW> sr;
+            ac_fetch_slice<SH::KW>(sr, a.in, VT_DIM, a.gain);
+            ac_issue<PH>(w0, wbase + u * unit_stride);
+            ac_slice_to_planes<true, SH::KW>(hi, lo, SH::PITCH, sr, red_ss);
+        } else {
+            ac_attn_regs ra;
+            ac_fetch_attn(ra, a.in);
+            ac_issue<PH>(w0, wbase + u * unit_stride);
             f32x4 *kvl = reinterpret_cast<f32x4 *>(ac_lds + 2 * SH::PLANE + SH::RED_BYTES);
             ac_stage_kv(kvl, ra);
             __syncthreads();
             ac_attention_to_planes(hi, lo, SH::PITCH, ra, kvl);
-        } else ac_rows_to_planes<true>(hi, lo, SH::PITCH, rr, red_ss);
-        __syncthreads();
+            __syncthreads();
+        }
         /* The request for unit u + G is never issued under a condition of its own: the compiler
          * counts outstanding loads statically, and behind a conditional request it would make the
          * product of unit u wait for unit u + G as well (which is what the two register sets are
@@ -351,7 +362,7 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
             if (nx >= n_units) {
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w0, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
+                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev, scale_ss);
                 break;
             }
             {
@@ -359,14 +370,14 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
                 __builtin_amdgcn_sched_barrier(0);
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w0, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
+                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev, scale_ss);
                 u = nx;
             }
             nx = u + G;
             if (nx >= n_units) {
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w1, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
+                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev, scale_ss);
                 break;
             }
             {
@@ -374,30 +385,29 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
                 __builtin_amdgcn_sched_barrier(0);
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w1, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
+                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev, scale_ss);
                 u = nx;
             }
         }
     } else {
         for (; u < n_units; u += G) {
             const uint16_t *wp = wbase + u * unit_stride;
-            ac_rows_regs rr;
-            ac_fetch_rows(rr, a.in, VT_FFN, NULL);
+            if (u != first_unit) __syncthreads();       /* nobody still reads red */
+            ac_slice_regs<SH::KW> sr;
+            ac_fetch_slice<SH::KW>(sr, a.in, VT_FFN, NULL);
             u32x4 wreg[2][SH::NL];
             ac_issue<PH>(wreg[0], wp);
             f32x4 ah = zero4, al = zero4;
 #pragma unroll
             for (int pass = 0; pass < SH::NPASS; pass++) {
-                __syncthreads();                        /* nobody still reads the planes or red */
-                ac_rows_to_planes<false>(hi, lo, SH::PITCH, rr, red_ss);
-                __syncthreads();
+                ac_slice_to_planes<false, SH::KW>(hi, lo, SH::PITCH, sr, red_ss);
                 if (pass + 1 < SH::NPASS) {
-                    ac_fetch_rows(rr, a.in + (pass + 1) * SH::KP, VT_FFN, NULL);
+                    ac_fetch_slice<SH::KW>(sr, a.in + (pass + 1) * SH::KP, VT_FFN, NULL);
                     ac_issue<PH>(wreg[(pass + 1) & 1], wp + (pass + 1) * SH::KP);
                 }
                 ac_consume(wreg[pass & 1], fa, fl, ah, al);
             }
-            ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev);
+            ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, u == first_unit, prev, nullptr);
         }
     }
 }
