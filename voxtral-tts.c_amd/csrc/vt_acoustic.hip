@@ -143,17 +143,18 @@ __device__ __forceinline__ void ac_slice_to_planes(unsigned char *hi, unsigned c
  * planes that feed the output projection (tts_bidirectional_attention,
  * voxtral_tts_kernels.c:467-525).  8 lanes per (branch, head), 16 dims each.  Every
  * lane keeps its q in registers; k and v, which the 4 heads of a group share, are
- * fetched once per workgroup (k|v are 2048 consecutive floats of a row) and handed
- * round through LDS: each head fetching its own copy made this kernel pull 295 KB
- * of activations through its CU instead of 147 KB. */
+ * fetched once and handed round through LDS: each head fetching its own copy made this
+ * kernel pull 295 KB of activations through its CU instead of 147 KB.
+ * Wave w serves the query heads 4 w .. 4 w + 3 of both branches, i.e. kv head w: their outputs are exactly
+ * the plane columns 512 w .. of the wave's own K slice, and the k|v rows they share are the wave's alone. */
 __device__ __forceinline__ void ac_fetch_attn(ac_attn_regs &r, const float *qkv) {
-    const int lane = vt_lane(), pair = vt_wave() * 8 + (lane >> 3), sub = lane & 7;
-    const int br = pair >> 5, h = pair & 31, d0 = sub * 16;
-    constexpr int ROW4 = 2 * VT_KV_DIM / 4;                    /* 16-byte groups of k|v per row */
+    const int lane = vt_lane(), wave = vt_wave(), p = lane >> 3, sub = lane & 7;
+    const int br = p >> 2, h = 4 * wave + (p & 3), d0 = sub * 16;
 #pragma unroll
-    for (int j = 0; j < AC_ROWS * ROW4 / AC_THREADS; j++) {
-        const int i = (int)threadIdx.x + AC_THREADS * j;
-        r.kv[j] = *reinterpret_cast<const f32x4 *>(qkv + (size_t)(i / ROW4) * VT_QKV_DIM + VT_Q_DIM + 4 * (i % ROW4));
+    for (int j = 0; j < AC_ROWS; j++) {                         /* row j: k (32 groups of 4) | v (32 groups) of kv head `wave` */
+        const int which = lane >> 5, g4 = lane & 31;
+        r.kv[j] = *reinterpret_cast<const f32x4 *>(qkv + (size_t)j * VT_QKV_DIM + VT_Q_DIM + which * VT_KV_DIM +
+                                                   wave * VT_HEAD_DIM + 4 * g4);
     }
 #pragma unroll
     for (int i = 0; i < 3; i++) {
@@ -163,26 +164,29 @@ __device__ __forceinline__ void ac_fetch_attn(ac_attn_regs &r, const float *qkv)
     }
 }
 
-/* k|v of the 6 rows into LDS as [row][2048] */
+/* the wave's k|v into its part of LDS as [row][k 32 | v 32] groups of 4 */
 __device__ __forceinline__ void ac_stage_kv(f32x4 *kvl, const ac_attn_regs &r) {
+    f32x4 *mine = kvl + vt_wave() * (AC_ROWS * 64);
 #pragma unroll
-    for (int j = 0; j < AC_ROWS * 2 * VT_KV_DIM / 4 / AC_THREADS; j++) kvl[(int)threadIdx.x + AC_THREADS * j] = r.kv[j];
+    for (int j = 0; j < AC_ROWS; j++) mine[j * 64 + vt_lane()] = r.kv[j];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");       /* LDS serves a wave in order */
+    __builtin_amdgcn_wave_barrier();
 }
 
 __device__ __forceinline__ void ac_attention_to_planes(unsigned char *hi, unsigned char *lo, int pitch,
                                                        const ac_attn_regs &r, const f32x4 *kvl) {
-    const int lane = vt_lane(), pair = vt_wave() * 8 + (lane >> 3), sub = lane & 7;
-    const int br = pair >> 5, h = pair & 31, d0 = sub * 16;
+    const int lane = vt_lane(), wave = vt_wave(), p = lane >> 3, sub = lane & 7;
+    const int br = p >> 2, h = 4 * wave + (p & 3), d0 = sub * 16;
     const float scale = 1.0f / sqrtf((float)VT_HEAD_DIM);
-    constexpr int ROW4 = 2 * VT_KV_DIM / 4;
+    const f32x4 *mine = kvl + wave * (AC_ROWS * 64);
     f32x4 k[3][4], v[3][4];
 #pragma unroll
     for (int j = 0; j < 3; j++)
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const int at = (br * 3 + j) * ROW4 + ((h >> 2) * VT_HEAD_DIM + d0) / 4 + e;
-            k[j][e] = kvl[at];
-            v[j][e] = kvl[at + VT_KV_DIM / 4];
+            const int at = (br * 3 + j) * 64 + d0 / 4 + e;
+            k[j][e] = mine[at];
+            v[j][e] = mine[at + 32];
         }
 #pragma unroll
     for (int i = 0; i < 3; i++) {
@@ -348,9 +352,9 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
             ac_issue<PH>(w0, wbase + u * unit_stride);
             f32x4 *kvl = reinterpret_cast<f32x4 *>(ac_lds + 2 * SH::PLANE + SH::RED_BYTES);
             ac_stage_kv(kvl, ra);
-            __syncthreads();
             ac_attention_to_planes(hi, lo, SH::PITCH, ra, kvl);
-            __syncthreads();
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
         /* The request for unit u + G is never issued under a condition of its own: the compiler
          * counts outstanding loads statically, and behind a conditional request it would make the
