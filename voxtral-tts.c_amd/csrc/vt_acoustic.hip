@@ -58,7 +58,10 @@ template <int PH> struct ac_shape {
     static constexpr int NL = KW / 32;                               /* 16-byte loads per lane and pass */
     static constexpr int PITCH = KP * 2 + 16;                        /* bytes per plane row */
     static constexpr int PLANE = AC_ROWS * PITCH;
-    static constexpr int RED_BYTES = 4 * (2 * AC_WAVES * AC_ROWS * 16 + AC_WAVES * 8);
+    /* units a workgroup takes on a 256-workgroup grid (more on a smaller one: then the buffers are reused) */
+    static constexpr int UNITS = PH == AC_W13 ? 6 : PH == AC_QKV ? 2 : 1;
+    static constexpr int RED_UNIT = AC_WAVES * AC_ROWS * 16;          /* floats: one unit's partial sums of all waves */
+    static constexpr int RED_BYTES = 4 * (UNITS * RED_UNIT + AC_WAVES * 8);
     /* attention + output projection: the k|v columns of the 6 rows, shared by the 4 heads of a group */
     static constexpr int KV_BYTES = PH == AC_WO ? AC_ROWS * 2 * VT_KV_DIM * 4 : 0;
     static constexpr int LDS_BYTES = 2 * PLANE + RED_BYTES + KV_BYTES;
@@ -263,10 +266,8 @@ __device__ __forceinline__ float ac_inv_rms_of(const float *red_ss, int m) {
     return 1.0f / sqrtf(tot / (float)VT_DIM + VT_EPS);
 }
 
-template <int PH>
-__device__ __forceinline__ void ac_finish_unit(const ac_phase_args &a, float *red, int n0, f32x4 acc_hi,
-                                               f32x4 acc_lo, bool have_prev = false, float prev = 0.f,
-                                               const float *red_ss = nullptr) {
+/* A wave leaves its partial sums of one unit in that unit's buffer; nobody waits. */
+__device__ __forceinline__ void ac_park_unit(float *red, f32x4 acc_hi, f32x4 acc_lo) {
     const int lane = vt_lane(), wave = vt_wave(), col = lane & 15, kg = lane >> 4;
     /* accumulator element v of lane l: activation row 4*(l/16) + v, weight row l%16 */
 #pragma unroll
@@ -274,31 +275,44 @@ __device__ __forceinline__ void ac_finish_unit(const ac_phase_args &a, float *re
         const int m = 4 * kg + v;
         if (m < AC_ROWS) red[(wave * AC_ROWS + m) * 16 + col] = acc_hi[v] + acc_lo[v];
     }
-    __syncthreads();
-    const int t = (int)threadIdx.x;
-    if (PH == AC_W13) {
-        if (t < AC_ROWS * 8 && (t & 7) < AC_RB / 2) {
-            const int m = t >> 3, j = t & 7;
-            float g = 0.f, u = 0.f;
+}
+
+/* Behind the workgroup's barrier: cross-wave sums and epilogues of the `n` units parked in red (unit j of
+ * them is weight rows (u0 + j * G) * 12 ..).  Thread t takes output element t % E of unit t / E. */
+template <int PH>
+__device__ __forceinline__ void ac_finish_units(const ac_phase_args &a, const float *red, int n, int u0, int G,
+                                                bool have_prev, float prev, const float *red_ss) {
+    typedef ac_shape<PH> SH;
+    constexpr int E = PH == AC_W13 ? AC_ROWS * 8 : AC_ROWS * 16;     /* threads per unit */
+    for (int t = (int)threadIdx.x; t < n * E; t += AC_THREADS) {
+        const int j = t / E, e = t % E;
+        const float *r = red + j * SH::RED_UNIT;
+        const int n0 = (u0 + j * G) * AC_RB;
+        if (PH == AC_W13) {
+            if ((e & 7) < AC_RB / 2) {
+                const int m = e >> 3, c = e & 7;
+                float g = 0.f, u = 0.f;
 #pragma unroll
-            for (int w = 0; w < AC_WAVES; w++) {
-                g += red[(w * AC_ROWS + m) * 16 + 2 * j];
-                u += red[(w * AC_ROWS + m) * 16 + 2 * j + 1];
+                for (int w = 0; w < AC_WAVES; w++) {
+                    g += r[(w * AC_ROWS + m) * 16 + 2 * c];
+                    u += r[(w * AC_ROWS + m) * 16 + 2 * c + 1];
+                }
+                const float inv = ac_inv_rms_of(red_ss, m);
+                g = __fmul_rn(g, inv);
+                u = __fmul_rn(u, inv);
+                a.out[(size_t)m * VT_FFN + (n0 >> 1) + c] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
             }
-            if (red_ss) { const float inv = ac_inv_rms_of(red_ss, m); g = __fmul_rn(g, inv); u = __fmul_rn(u, inv); }
-            a.out[(size_t)m * VT_FFN + (n0 >> 1) + j] = __fmul_rn(__fdiv_rn(g, __fadd_rn(1.0f, expf(-g))), u);
-        }
-    } else if (t < AC_ROWS * 16 && (t & 15) < AC_RB) {
-        const int m = t >> 4, n = t & 15;
-        float y = 0.f;
+        } else if ((e & 15) < AC_RB) {
+            const int m = e >> 4, c = e & 15;
+            float y = 0.f;
 #pragma unroll
-        for (int w = 0; w < AC_WAVES; w++) y += red[(w * AC_ROWS + m) * 16 + n];
-        if (PH == AC_QKV) {
-            if (red_ss) y = __fmul_rn(y, ac_inv_rms_of(red_ss, m));
-            a.out[(size_t)m * VT_QKV_DIM + n0 + n] = y;
-        } else {
-            float *p = a.out + (size_t)m * VT_DIM + n0 + n;
-            *p = __fadd_rn(have_prev ? prev : *p, y);
+            for (int w = 0; w < AC_WAVES; w++) y += r[(w * AC_ROWS + m) * 16 + c];
+            if (PH == AC_QKV) {
+                a.out[(size_t)m * VT_QKV_DIM + n0 + c] = __fmul_rn(y, ac_inv_rms_of(red_ss, m));
+            } else {
+                float *p = a.out + (size_t)m * VT_DIM + n0 + c;
+                *p = __fadd_rn(have_prev && j == 0 ? prev : *p, y);
+            }
         }
     }
 }
@@ -309,8 +323,8 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
     typedef ac_shape<PH> SH;
     extern __shared__ __attribute__((aligned(16))) unsigned char ac_lds[];
     unsigned char *hi = ac_lds, *lo = ac_lds + SH::PLANE;
-    float *red = reinterpret_cast<float *>(ac_lds + 2 * SH::PLANE);          /* 2 x [8 waves][6][16] */
-    float *red_ss = red + 2 * AC_WAVES * AC_ROWS * 16;                       /* [8 waves][8] */
+    float *red = reinterpret_cast<float *>(ac_lds + 2 * SH::PLANE);          /* UNITS x [8 waves][6][16] */
+    float *red_ss = red + SH::UNITS * SH::RED_UNIT;                          /* [8 waves][8] */
     const int lane = vt_lane(), wave = vt_wave();
     const int col = lane & 15, kg = lane >> 4;
     const bool live = col < AC_RB;
@@ -339,6 +353,15 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
 
     /* behind an RMSNorm the planes hold x * gain; the epilogue multiplies by 1/rms(x) */
     const float *scale_ss = (PH == AC_QKV || PH == AC_W13) ? red_ss : nullptr;
+    constexpr bool RES = PH == AC_WO || PH == AC_W2;
+    int k = 0, u0 = u;                                  /* units parked, and the first of them */
+    auto flush = [&] {
+        __syncthreads();
+        ac_finish_units<PH>(a, red, k, u0, G, RES && u0 == first_unit, prev, scale_ss);
+        __syncthreads();                                /* the buffers are free again */
+        u0 += k * G;
+        k = 0;
+    };
     if (SH::NPASS == 1) {
         if (PH != AC_WO) {
             /* every wave for itself: its K slice of the rows, no workgroup barrier before the products */
@@ -359,14 +382,16 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
         /* The request for unit u + G is never issued under a condition of its own: the compiler
          * counts outstanding loads statically, and behind a conditional request it would make the
          * product of unit u wait for unit u + G as well (which is what the two register sets are
-         * there to avoid).  The last unit of a workgroup takes the branch without a request. */
-        float *red1 = red + AC_WAVES * AC_ROWS * 16;
+         * there to avoid).  The last unit of a workgroup takes the branch without a request.
+         * A wave parks its partial sums of a unit in that unit's buffer and goes on: the waves of a
+         * workgroup meet once, behind the last unit (or when all buffers are full, on a small grid). */
         for (;;) {
             int nx = u + G;
             if (nx >= n_units) {
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w0, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev, scale_ss);
+                ac_park_unit(red + k * SH::RED_UNIT, ah, al);
+                k++;
                 break;
             }
             {
@@ -374,14 +399,16 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
                 __builtin_amdgcn_sched_barrier(0);
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w0, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev, scale_ss);
+                ac_park_unit(red + k * SH::RED_UNIT, ah, al);
+                if (++k == SH::UNITS) flush();
                 u = nx;
             }
             nx = u + G;
             if (nx >= n_units) {
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w1, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev, scale_ss);
+                ac_park_unit(red + k * SH::RED_UNIT, ah, al);
+                k++;
                 break;
             }
             {
@@ -389,14 +416,14 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
                 __builtin_amdgcn_sched_barrier(0);
                 f32x4 ah = zero4, al = zero4;
                 ac_consume(w1, fa, fl, ah, al);
-                ac_finish_unit<PH>(a, red1, u * AC_RB, ah, al, (PH == AC_WO || PH == AC_W2) && u == first_unit, prev, scale_ss);
+                ac_park_unit(red + k * SH::RED_UNIT, ah, al);
+                if (++k == SH::UNITS) flush();
                 u = nx;
             }
         }
     } else {
         for (; u < n_units; u += G) {
             const uint16_t *wp = wbase + u * unit_stride;
-            if (u != first_unit) __syncthreads();       /* nobody still reads red */
             ac_slice_regs<SH::KW> sr;
             ac_fetch_slice<SH::KW>(sr, a.in, VT_FFN, NULL);
             u32x4 wreg[2][SH::NL];
@@ -411,8 +438,13 @@ vt_ac_phase_kernel(ac_phase_args a, int n_units) {
                 }
                 ac_consume(wreg[pass & 1], fa, fl, ah, al);
             }
-            ac_finish_unit<PH>(a, red, u * AC_RB, ah, al, u == first_unit, prev, nullptr);
+            ac_park_unit(red + k * SH::RED_UNIT, ah, al);
+            if (++k == SH::UNITS) flush();
         }
+    }
+    if (k) {
+        __syncthreads();
+        ac_finish_units<PH>(a, red, k, u0, G, RES && u0 == first_unit, prev, scale_ss);
     }
 }
 
