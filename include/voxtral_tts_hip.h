@@ -298,9 +298,10 @@ const char *tts_hip_last_error(void);
 void tts_hip_timer_start(void);
 float tts_hip_timer_stop_ms(void);
 /* Average duration in ms of one launch of a single kernel, timed with events on the
- * internal stream over `iters` launches on zero-filled work buffers (needs the weights
- * uploaded; launch i takes the weights of uploaded layer i modulo their number, so that they
- * come from HBM as in a real pass): which 0..3 = sequence-level product at M = 512 with the
+ * internal stream over `iters` launches on pseudo-random activations of normal size (on zeros
+ * the matrix cores draw less power and the products measure 5-15 % faster than in a real pass;
+ * needs the weights uploaded; launch i takes the weights of uploaded layer i modulo their
+ * number, so that they come from HBM as in a real pass): which 0..3 = sequence-level product at M = 512 with the
  * q|k|v, output, gate/up and down projection; 4 = causal attention at 512 queries (KV cache
  * of at least 512 rows); 10..13 = the four acoustic phase kernels, 14 = the four of them in
  * order on one layer (the value is the duration of all four); 20..23 = the codec's fp32

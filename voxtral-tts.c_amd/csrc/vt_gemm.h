@@ -17,7 +17,7 @@ void vt_launch_gemm(float *d_C, const uint16_t *d_Ahi, const uint16_t *d_Alo, co
 void vt_launch_gemm_ex(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
                        const uint16_t *d_W, int M, int N, int K, int splits);
 /* The same product on the 128 x 256 tile kernel, which reads the weights in fragment order
- * (vt_launch_frag_layout): N % 256 == 0, K % 64 == 0, an even number of 64-wide K steps per cut. */
+ * (vt_launch_frag_layout): N % 256 == 0, K % 128 == 0, at most K / 128 cuts (they need not divide K). */
 int vt_gemm_frag_shape_ok(int N, int K, int splits);
 void vt_launch_gemm_frag(float *d_C, int ldc, size_t plane_stride, const uint16_t *d_Ahi, const uint16_t *d_Alo,
                          const uint16_t *d_Wf, int M, int N, int K, int splits);
@@ -41,6 +41,8 @@ void vt_launch_residual_norm_split(float *d_x, const float *d_part, int splits, 
 /* n_out a multiple of 4, tail_col0 of 8: planes of silu(gate)*up from interleaved (gate, up) pairs */
 void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, size_t n_out, int tail_col0,
                             const float *d_tail, int tail_planes, size_t tail_stride);
+/* benchmark input: n pseudo-random bf16 values per plane (d_lo may be NULL) */
+void vt_launch_bench_fill(uint16_t *d_hi, uint16_t *d_lo, size_t n);
 void vt_launch_sum_planes(float *d_out, const float *d_part, int splits, size_t stride, size_t n);
 
 #endif /* VT_GEMM_H */

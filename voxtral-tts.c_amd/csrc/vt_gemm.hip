@@ -181,7 +181,9 @@ vt_gemm_mfma_kernel(float *C, const uint16_t *Ahi, const uint16_t *Alo, const ui
  * apart, and the CU's address pipeline, not the matrix cores, sets the pace (measured: 434 against
  * 518 TFLOP/s).  The backbone therefore keeps a second copy of its matrices in fragment order,
  * written once at upload by vt_frag_layout_kernel: every load is then 1 KB of consecutive bytes.
- * Needs N % 256 == 0, K % 64 == 0 and an even number of K steps per cut. */
+ * Needs N % 256 == 0 and K % 128 == 0: a cut is a whole number of pairs of K steps, and the cuts of one
+ * product may differ by one pair (64 steps in 5 cuts: 14, 14, 12, 12, 12), so that the cut count can be
+ * chosen to fill the CUs (48 tiles x 5 = 240 items) rather than to divide K. */
 #define GW_TM 128
 #define GW_TN 256
 #define GW_PLANE (GW_TM * GM_ROWB)
@@ -199,7 +201,7 @@ struct gw_part {
     float *C;                /* output of this set: `splits` planes, plane_stride floats apart, row pitch ldc */
     const uint16_t *Wf;      /* fragment-order weights of the set's first column */
     size_t plane_stride;
-    int ldc, n_tiles, splits, k_split;
+    int ldc, n_tiles, splits, k_pairs;   /* k_pairs: K / 128, dealt out over the `splits` cuts */
     /* gate|up product in the paired column order (vt_launch_frag_layout with pair = 1): instead of C, the
      * (hi, lo) planes of SiLU(gate) * up, row pitch ldh; the set's first column is h column h_col0 */
     uint16_t *h_hi, *h_lo;
@@ -213,31 +215,22 @@ vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int 
     const int id = (int)blockIdx.x;
   for (int pi = 0; pi < plan.n_parts; pi++) {
     const gw_part &P = plan.part[pi];
-    const int n_tiles = P.n_tiles, k_split = P.k_split, ldc = P.ldc;
-    if (id >= m_tiles * n_tiles * P.splits) continue;
+    const int n_tiles = P.n_tiles, ldc = P.ldc, items = m_tiles * n_tiles * P.splits;
+    if (id >= items) continue;
     float *C = P.C;
     const uint16_t *Wf = P.Wf;
     const size_t plane_stride = P.plane_stride;
-    int mt, nt, sp;
-    if (((n_tiles * P.splits) & 7) == 0) {
-        /* Slot id lands on XCD id % 8.  An XCD takes all M tiles of a run of consecutive (K cut, N tile)
-         * pairs: the M tiles of a pair share its weights, the N tiles of a K cut share the activation
-         * planes of that cut, and both then leave the memory side once per XCD instead of once per
-         * workgroup (the two slices are the same size: 128 rows x 4 bytes against 256 rows x 2 bytes). */
-        const int x = id & 7, q = id >> 3, per_xcd = (n_tiles * P.splits) >> 3;
-        const int ci = x * per_xcd + q / m_tiles;
-        mt = q % m_tiles;
-        nt = ci % n_tiles;
-        sp = ci / n_tiles;
-    } else {
-        const int r = id / m_tiles;
-        mt = id % m_tiles;
-        nt = r % n_tiles;
-        sp = r / n_tiles;
-    }
+    /* Slot id lands on XCD id % 8.  An XCD takes a run of consecutive items, M tile fastest, then N tile,
+     * then K cut: the M tiles of a (K cut, N tile) pair share its weights, the N tiles of a K cut share the
+     * activation planes of that cut, and both then leave the memory side once per XCD instead of once per
+     * workgroup (the two slices are the same size: 128 rows x 4 bytes against 256 rows x 2 bytes). */
+    const int li = (items & 7) == 0 ? (id & 7) * (items >> 3) + (id >> 3) : id;
+    const int mt = li % m_tiles, ci = li / m_tiles, nt = ci % n_tiles, sp = ci / n_tiles;
     const int t = (int)threadIdx.x, lane = t & 63, wave = t >> 6;
     const int lr = t >> 3, lc = t & 7;               /* staging: row lr + 32 i, 16-byte chunk lc */
-    const int k0 = sp * k_split, tiles = k_split / GM_BK;
+    /* K is dealt out in pairs of 64-wide steps; the first k_pairs % splits cuts take one pair more */
+    const int pq = P.k_pairs / P.splits, pr = P.k_pairs % P.splits;
+    const int k0 = 2 * GM_BK * (sp * pq + (sp < pr ? sp : pr)), tiles = 2 * (pq + (sp < pr ? 1 : 0));
 
     /* rows past M read row 0 of the tile again: their products land in accumulator rows that are
      * never stored (the rows of a matrix instruction do not mix), so nothing has to be zeroed */
@@ -416,7 +409,7 @@ vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int 
 static int gm_blocks(size_t n);
 
 int vt_gemm_frag_shape_ok(int N, int K, int splits) {
-    return N % GW_TN == 0 && K % GM_BK == 0 && splits >= 1 && K % splits == 0 && (K / splits) % (2 * GM_BK) == 0;
+    return N % GW_TN == 0 && K % (2 * GM_BK) == 0 && splits >= 1 && splits <= K / (2 * GM_BK);
 }
 
 static int gw_ready(void) {
@@ -436,7 +429,7 @@ void vt_launch_gemm_frag(float *d_C, int ldc, size_t plane_stride, const uint16_
     const int m_tiles = (M + GW_TM - 1) / GW_TM;
     gw_plan plan = {};
     plan.n_parts = 1;
-    plan.part[0] = gw_part{d_C, d_Wf, plane_stride, ldc, N / GW_TN, splits, K / splits, NULL, NULL, 0, 0};
+    plan.part[0] = gw_part{d_C, d_Wf, plane_stride, ldc, N / GW_TN, splits, K / (2 * GM_BK), NULL, NULL, 0, 0};
     hipLaunchKernelGGL(vt_gemm_wide_kernel, dim3(m_tiles * (N / GW_TN) * splits), dim3(256), GW_LDS, g_vt.stream,
                        plan, d_Ahi, d_Alo, M, K, m_tiles);
 }
@@ -452,11 +445,11 @@ void vt_launch_gemm_frag_swiglu(uint16_t *d_hhi, uint16_t *d_hlo, int ldh, float
     const int m_tiles = (M + GW_TM - 1) / GW_TM;
     gw_plan plan = {};
     plan.n_parts = n_tail > 0 ? 2 : 1;
-    plan.part[0] = gw_part{NULL, d_Wf, 0, 0, n_main / GW_TN, 1, K, d_hhi, d_hlo, ldh, 0};
+    plan.part[0] = gw_part{NULL, d_Wf, 0, 0, n_main / GW_TN, 1, K / (2 * GM_BK), d_hhi, d_hlo, ldh, 0};
     int items = m_tiles * (n_main / GW_TN);
     if (n_tail > 0) {
         plan.part[1] = gw_part{d_tail, d_Wf + (size_t)n_main * K, (size_t)M * n_tail, n_tail, n_tail / GW_TN, tail_splits,
-                               K / tail_splits, NULL, NULL, 0, 0};
+                               K / (2 * GM_BK), NULL, NULL, 0, 0};
         const int items1 = m_tiles * (n_tail / GW_TN) * tail_splits;
         if (items1 > items) items = items1;
     }
@@ -678,4 +671,21 @@ __global__ void vt_sum_planes_kernel(float *out, const float *part, int splits, 
 void vt_launch_sum_planes(float *d_out, const float *d_part, int splits, size_t stride, size_t n) {
     hipLaunchKernelGGL(vt_sum_planes_kernel, dim3(gm_blocks(n)), dim3(256), 0, g_vt.stream, d_out, d_part,
                        splits, stride, n);
+}
+
+/* Benchmark input: pseudo-random bf16 values of the size of normalised activations, hi in +-(2^-7 .. 2) and
+ * (d_lo != NULL) lo 2^-9 of that with a mantissa of its own.  Written over a float array as 2 n halves it
+ * gives floats of the same range. */
+__global__ void vt_bench_fill_kernel(uint16_t *hi, uint16_t *lo, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        unsigned h = (unsigned)i * 2654435761u + 12345u;
+        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+        /* sign, an exponent in 120..127 (2^-7 .. 1, times 1.x), 7 mantissa bits */
+        hi[i] = (uint16_t)(((h & 1u) << 15) | ((120u + ((h >> 1) & 7u)) << 7) | ((h >> 4) & 127u));
+        if (lo) lo[i] = (uint16_t)((((h >> 11) & 1u) << 15) | ((111u + ((h >> 1) & 7u)) << 7) | ((h >> 12) & 127u));
+    }
+}
+
+void vt_launch_bench_fill(uint16_t *d_hi, uint16_t *d_lo, size_t n) {
+    hipLaunchKernelGGL(vt_bench_fill_kernel, dim3(gm_blocks(n)), dim3(256), 0, g_vt.stream, d_hi, d_lo, n);
 }

@@ -393,6 +393,12 @@ void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, c
 #define VT_W13_TAIL_CUT 4
 #endif
 
+/* K cuts of a product of `tiles` output tiles: one item per CU at most, `most` planes at most */
+static int vt_prefill_cuts(int tiles, int most) {
+    const int c = g_vt.n_cu / tiles;
+    return c < 1 ? 1 : c > most ? most : c;
+}
+
 static int ew_blocks(size_t n) { size_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : b); }
 
 extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int start_pos, float *out_x) {
@@ -405,10 +411,13 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
     const size_t S = (size_t)seq_len;
     hipStream_t st = g_vt.stream;
     /* work area: x | wide f32 (qkv or gate/up) | q | partial planes | hi | lo */
-    /* K is cut so that every product launches about two workgroups per CU (M tiles x N tiles x
-     * cuts): 4 M tiles at 512 rows give 192 / 96 / 96 tiles for q|k|v / output / down */
+    /* K is cut into as many ranges as give every CU at most one item (M tiles x N tiles x cuts; the cuts
+     * need not divide K): 4 M tiles at 512 rows are 96 / 48 / 48 tiles for q|k|v / output / down, i.e.
+     * 192 / 240 / 240 items */
     const int m_tiles = (seq_len + 127) / 128;
-    const int sp_qkv = m_tiles >= 3 ? 2 : 4, sp_wo = m_tiles >= 3 ? 4 : 8, sp_w2 = m_tiles >= 3 ? 4 : 8;
+    const int fq = vt_prefill_cuts(m_tiles * (VT_QKV_DIM / 256), 4), fo = vt_prefill_cuts(m_tiles * (VT_DIM / 256), 8);
+    /* the 128 x 128 kernel on row-major weights (layers without a fragment copy) wants cuts that divide K */
+    const int rq = m_tiles >= 3 ? 2 : 4, ro = m_tiles >= 3 ? 4 : 8;
     const int tail_cols = m_tiles == 4 ? 16 * 128 : 0;      /* part holds 4 x S x 2048 <= 8 x S x 3072 */
     const size_t n_x = S * VT_DIM, n_wide = S * 4 * VT_QKV_DIM, n_q = S * VT_Q_DIM, n_part = 8 * S * VT_DIM;
     const size_t n_plane = S * VT_FFN;                            /* bf16 elements per plane */
@@ -427,6 +436,7 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         float *vc = g_hip.kv_cache_v_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
         const vt_layer_frag *F = &g_vt.h_frag[l];
         const bool frag = F->wqkv && F->wo && F->w13 && F->w2;
+        const int sp_qkv = frag ? fq : rq, sp_wo = frag ? fo : ro, sp_w2 = sp_wo;
         if (frag) vt_launch_gemm_frag(wide, VT_QKV_DIM, S * VT_QKV_DIM, hi, lo, F->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
         else vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
         /* k (rotated) and v into the cache; the attention takes q from the product's planes itself */
@@ -482,7 +492,8 @@ extern "C" void tts_hip_llm_prefill(const float *embeds, int seq_len, int start_
  * every launch on the next acoustic layer; 14: the four phase launches of one acoustic layer
  * in order (the value is the time of all four).
  * Returns the average duration of one launch in ms (events on the internal stream), or
- * a negative value on error.  Buffers hold zeros: the kernels are data-independent. */
+ * a negative value on error.  The activation planes (and q) hold pseudo-random values of the size of
+ * normalised activations; the attention reads whatever the KV cache of layer 0 holds. */
 float vt_bench_acoustic_phase(int phase, int iters);
 
 extern "C" float tts_hip_bench_kernel(int which, int iters) {
@@ -492,8 +503,10 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
     if (which < 0 || which > 4 || g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_bench_kernel: unknown kernel %d", which); return -1.f; }
     const int S = 512;
     if (which == 4 && g_vt.kv_max < S) { vt_set_error("tts_hip_bench_kernel: KV cache shorter than 512"); return -1.f; }
-    static const int NN[4] = {VT_QKV_DIM, VT_DIM, 2 * VT_FFN, VT_DIM}, KK[4] = {VT_DIM, VT_Q_DIM, VT_DIM, VT_FFN},
-                     SP[4] = {2, 4, 1, 4};
+    static const int NN[4] = {VT_QKV_DIM, VT_DIM, 2 * VT_FFN, VT_DIM}, KK[4] = {VT_DIM, VT_Q_DIM, VT_DIM, VT_FFN};
+    const int SP[4] = {vt_prefill_cuts(4 * (VT_QKV_DIM / 256), 4), vt_prefill_cuts(4 * (VT_DIM / 256), 8), 1,
+                       vt_prefill_cuts(4 * (VT_DIM / 256), 8)};
+    static const int RP[4] = {2, 4, 1, 4};            /* row-major weights: cuts that divide K */
     const size_t n_out = (size_t)S * 2 * VT_FFN * 4, n_plane = (size_t)S * VT_FFN, n_q = (size_t)S * VT_Q_DIM;
     const size_t bytes = sizeof(float) * (n_out + n_q) + 2 * sizeof(uint16_t) * n_plane;
     unsigned char *base = (unsigned char *)vt_scratch(bytes);
@@ -501,6 +514,14 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
     if (vt_check(hipMemsetAsync(base, 0, bytes, g_vt.stream), "bench clear")) return -1.f;
     float *out = (float *)base, *q = out + n_out;
     uint16_t *hi = (uint16_t *)(q + n_q), *lo = hi + n_plane;
+    /* The kernels do the same work on any data, but not at the same clock: on planes of zeros the matrix
+     * cores draw less power and the products measure 5-15 % faster than inside a prefill.  The planes get
+     * values of the size a normalised activation has: hi = bf16 of a uniform value in (-2, 2), lo a value
+     * 2^-9 of that with its own mantissa. */
+    if (which < 4)
+        vt_launch_bench_fill(hi, lo, n_plane);
+    else                                              /* q: floats whose upper halves are such bf16 values */
+        vt_launch_bench_fill((uint16_t *)q, NULL, 2 * n_q);
     float ms = -1.f;
     for (int it = -2; it < iters; it++) {
         if (it == 0 && vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench start")) return -1.f;
@@ -522,7 +543,7 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
             vt_launch_gemm_ex(out + (size_t)S * 2 * VT_FFN, tail, (size_t)S * tail, hi, lo,
                               W[2] + (size_t)main_cols * VT_DIM, S, tail, VT_DIM, 4);
         } else if (which < 4 && frag) vt_launch_gemm_frag(out, NN[which], (size_t)S * NN[which], hi, lo, Wf[which], S, NN[which], KK[which], SP[which]);
-        else if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], SP[which]);
+        else if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], RP[which]);
         else vt_launch_prefill_attention(out, NULL, NULL, q, VT_Q_DIM, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu, S, 0, VT_ATT_SCALE);
     }
     if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;
