@@ -189,3 +189,9 @@ def test_prefill_512_one_layer():
 
 def test_prefill_chunks_three_layers():
     _prefill_case(3, [150, 45, 1], 200, lambda n: range(0, n, 3))
+
+
+def test_prefill_row_counts_with_uneven_k_cuts():
+    """300 rows are 3 row tiles: the output and down products then run in 7 K cuts of 5 or 4 (11 or 10)
+    pairs of steps and q|k|v in 3; 650 rows (6 tiles) take 3 cuts and none."""
+    _prefill_case(1, [300, 650], 960, lambda n: range(0, n, 7))
