@@ -290,6 +290,11 @@ void tts_hip_set_decode_mode(int mode);
  * tts_hip_to_device, tts_hip_memset, tts_hip_timer_stop_ms (which then returns a negative time).
  * The report resets the barrier; the next step starts clean. */
 void tts_hip_set_barrier_timeout(unsigned long long ticks);
+/* Workgroups of the acoustic transformer's product kernels: 0 (the default) = one per CU, else
+ * 1 .. the CU count.  The results do not depend on it, bit for bit (a unit of 12 weight rows is summed the
+ * same way whichever workgroup takes it); a smaller grid leaves CUs to other work and makes a workgroup
+ * walk more units.  No counterpart in the reference. */
+void tts_hip_set_acoustic_grid(int workgroups);
 /* Number of failed calls since init, and the text of the last failure. */
 int tts_hip_error_count(void);
 const char *tts_hip_last_error(void);

@@ -147,6 +147,27 @@ def test_more_frames_against_oracle_with_margins(ac_session):
     assert mism <= 1
 
 
+def test_frame_does_not_depend_on_the_acoustic_grid(ac_session):
+    """On a smaller grid a workgroup of the product kernels walks more units: other loop tails (one,
+    two or three units left), parked partial sums flushed in between.  A unit is summed the same way
+    whichever workgroup takes it, so latent and codes are the same bit for bit."""
+    hip, orc, ac = ac_session
+    h, x0 = S.f32_normal(S.DIM, 77), S.f32_normal(S.ACOUSTIC_DIM, 78)
+    ref_codes, ref_x = hip.acoustic_frame(h, x0)
+    try:
+        for grid in (100, 37, 7):
+            hip.lib.tts_hip_set_acoustic_grid(grid)
+            codes, x = hip.acoustic_frame(h, x0)
+            hip.check()
+            assert np.array_equal(codes, ref_codes), grid
+            assert np.array_equal(x.view(np.uint32), ref_x.view(np.uint32)), grid
+        hip.lib.tts_hip_set_acoustic_grid(100000)
+        assert "tts_hip_set_acoustic_grid" in hip.lib.tts_hip_last_error().decode()
+        hip.err0 = hip.lib.tts_hip_error_count()          # that failure was asked for
+    finally:
+        hip.lib.tts_hip_set_acoustic_grid(0)
+
+
 def test_end_audio_frame(ac_session):
     hip, orc, ac = ac_session
     ac2 = S.Acoustic(50)

@@ -658,7 +658,8 @@ static int launch_phase(const uint16_t *W, const float *in, const float *gain, f
     }
     ac_phase_args a = {W, in, gain, out};
     const int n_units = n_rows / AC_RB;
-    const int grid = n_units < g_vt.n_cu ? n_units : g_vt.n_cu;
+    const int most = g_vt.ac_grid > 0 && g_vt.ac_grid < g_vt.n_cu ? g_vt.ac_grid : g_vt.n_cu;
+    const int grid = n_units < most ? n_units : most;
     hipLaunchKernelGGL(vt_ac_phase_kernel<PH>, dim3(grid), dim3(AC_THREADS), lds, g_vt.stream, a, n_units);
     return 0;
 }

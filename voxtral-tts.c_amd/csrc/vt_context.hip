@@ -406,6 +406,13 @@ extern "C" void tts_hip_set_decode_mode(int mode) {
     g_vt.decode_mode = mode;
 }
 extern "C" void tts_hip_set_barrier_timeout(unsigned long long ticks) { g_vt.bar_timeout = ticks; }
+extern "C" void tts_hip_set_acoustic_grid(int workgroups) {
+    if (workgroups < 0 || (g_vt.initialized && workgroups > g_vt.n_cu)) {
+        vt_set_error("tts_hip_set_acoustic_grid: %d workgroups (0 or 1..%d)", workgroups, g_vt.n_cu);
+        return;
+    }
+    g_vt.ac_grid = workgroups;
+}
 extern "C" int tts_hip_error_count(void) { return g_vt.error_count; }
 extern "C" const char *tts_hip_last_error(void) { return g_vt.last_error; }
 

@@ -43,6 +43,7 @@ struct vt_state {
     int initialized;
     int device;
     int n_cu;
+    int ac_grid;                  /* workgroups of the acoustic product kernels; 0 = n_cu */
     int grid;                     /* workgroups of the persistent kernels */
     size_t step_dyn_lds;          /* dynamic LDS that pins one workgroup per CU */
     int step_checked, step_fits;  /* residency of the whole-step kernel's grid, asked once per context */
