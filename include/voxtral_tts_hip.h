@@ -290,6 +290,11 @@ void tts_hip_set_decode_mode(int mode);
  * tts_hip_to_device, tts_hip_memset, tts_hip_timer_stop_ms (which then returns a negative time).
  * The report resets the barrier; the next step starts clean. */
 void tts_hip_set_barrier_timeout(unsigned long long ticks);
+/* Workgroups of the backbone's whole-step decode kernel: 0 (the default) = the CU count rounded down to
+ * a multiple of 8, else a multiple of 8 from 72 up to that.  Waits for the library's stream.  Results
+ * agree to rounding, not bit for bit (the attention's key chunks follow the grid).  No counterpart in
+ * the reference. */
+void tts_hip_set_decode_grid(int workgroups);
 /* Workgroups of the acoustic transformer's product kernels: 0 (the default) = one per CU, else
  * 1 .. the CU count.  The results do not depend on it, bit for bit (a unit of 12 weight rows is summed the
  * same way whichever workgroup takes it); a smaller grid leaves CUs to other work and makes a workgroup

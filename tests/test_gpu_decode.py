@@ -72,6 +72,50 @@ def test_one_layer_decode_with_cached_positions(pos):
         hip.close()
 
 
+@pytest.mark.parametrize("pos", [300, 575, 1100, 4100])
+def test_one_layer_decode_on_smaller_grids(pos):
+    """The whole-step kernel deals rows, attention heads and key chunks by its grid size: the same
+    layer on 72, 128 and 200 workgroups (a device with fewer CUs), both schedules, at a position of
+    every attention schedule."""
+    kv_max = pos + 8
+    layer = S.Layer(3)
+    ones = np.ones(S.DIM, np.float32)
+    k = np.zeros((26, kv_max, S.KV_DIM), np.float32)
+    v = np.zeros((26, kv_max, S.KV_DIM), np.float32)
+    k[0, :pos] = S.f32_normal((pos, S.KV_DIM), 200)
+    v[0, :pos] = S.f32_normal((pos, S.KV_DIM), 300)
+    x = S.f32_normal(S.DIM, 42)
+    orc = cases.OracleBackend(threads=16)
+    orc.llm_open([layer], ones, kv_max, n_layers=1)
+    orc.kv_k[0], orc.kv_v[0] = k[0], v[0]
+    orc.pos = pos
+    ref_h = orc.llm_forward(x)
+    hip = H.Hip(kv_max=kv_max)
+    try:
+        hip.upload_decoder([layer], ones, 1)
+        hip.set_kv(k, v)
+        for grid in (72, 128, 200, 0):
+            hip.lib.tts_hip_set_decode_grid(grid)
+            hip.check()
+            for mode in (0, 1):
+                hip.lib.tts_hip_set_decode_mode(mode)
+                hip.pos = pos
+                got_h = hip.llm_forward(x)
+                assert_close(ref_h, got_h, f"hidden grid {grid} mode {mode}")
+                gk, gv = hip.kv()
+                assert_close(orc.kv_k[0, pos], gk[0, pos], "k row")
+                assert_close(orc.kv_v[0, pos], gv[0, pos], "v row")
+        for bad in (64, 100, 4096):
+            hip.lib.tts_hip_set_decode_grid(bad)
+            assert "tts_hip_set_decode_grid" in hip.lib.tts_hip_last_error().decode()
+        hip.err0 = hip.lib.tts_hip_error_count()          # those failures were asked for
+        hip.lib.tts_hip_set_decode_mode(0)
+        hip.pos = pos
+        assert_close(ref_h, hip.llm_forward(x), "after the refused grids")
+    finally:
+        hip.close()
+
+
 def test_schedules_agree_and_match_oracle_over_steps():
     """Mode 0 = persistent whole-step kernel, mode 1 = one kernel per phase.  Both run the same
     phase code and must agree bit for bit, run after run."""
@@ -113,6 +157,38 @@ def test_schedules_agree_and_match_oracle_over_steps():
         for l in range(n_layers):
             assert_close(orc.kv_k[l, :steps], gk[l, :steps], f"k cache layer {l}")
             assert_close(orc.kv_v[l, :steps], gv[l, :steps], f"v cache layer {l}")
+    finally:
+        hip.close()
+
+
+def test_five_layers_on_136_workgroups():
+    """Layer-to-layer hand-overs on a grid that is no power of two: teacher-forced steps against the
+    oracle, and the two schedules bit for bit."""
+    layers = [S.Layer(1), S.Layer(2), S.Layer(4)]
+    norm = S.norm_weight(S.DIM, 99)
+    n_layers, steps = 5, 4
+    orc = cases.OracleBackend(threads=16)
+    orc.llm_open(layers, norm, 32, n_layers=n_layers)
+    hip = H.Hip(kv_max=32)
+    try:
+        hip.upload_decoder(layers, norm, n_layers)
+        hip.lib.tts_hip_set_decode_grid(136)
+        hip.check()
+        refs, e = [], S.f32_normal(S.DIM, 6)
+        for s in range(steps):
+            refs.append(orc.llm_forward(e))
+            e = refs[-1].copy()
+        outs = {}
+        for mode in (0, 1):
+            hip.lib.tts_hip_set_decode_mode(mode)
+            hip.pos = 0
+            e, hs = S.f32_normal(S.DIM, 6), []
+            for s in range(steps):
+                hs.append(hip.llm_forward(e))
+                assert_close(refs[s], hs[-1], f"mode {mode} step {s}")
+                e = refs[s].copy()
+            outs[mode] = np.stack(hs)
+        assert np.array_equal(outs[0], outs[1])
     finally:
         hip.close()
 

@@ -123,6 +123,7 @@ SIGNATURES = {
     "tts_hip_generate_frame": (None, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]),
     "tts_hip_set_barrier_timeout": (None, [C.c_ulonglong]),
     "tts_hip_set_acoustic_grid": (None, [C.c_int]),
+    "tts_hip_set_decode_grid": (None, [C.c_int]),
     "tts_hip_upload_codec_weights": (C.c_int, [vp]),
     "tts_hip_codec_decode": (None, [vp, C.c_int, C.POINTER(f32p), i32p]),
     "tts_hip_codec_decode_device": (C.c_int, [vp, C.c_int, vp]),

@@ -316,6 +316,25 @@ static int step_aborted(int flag) {
     return -1;
 }
 
+/* Workgroups of the whole-step kernel: 0 = the default (the CU count rounded down to a multiple of the
+ * KV heads), else a multiple of 8 between 72 and that default.  The barrier's flags start from zero
+ * again, so workgroups that sat out a few steps do not come back with an old epoch. */
+extern "C" void tts_hip_set_decode_grid(int workgroups) {
+    if (!g_vt.initialized) { vt_set_error("tts_hip_set_decode_grid: backend not initialised"); return; }
+    const int full = g_vt.n_cu / VT_KV_HEADS * VT_KV_HEADS;
+    const int grid = workgroups == 0 ? full : workgroups;
+    if (grid > full || !grid_fits(grid)) {
+        vt_set_error("tts_hip_set_decode_grid: %d workgroups (0, or a multiple of %d in 72..%d)", workgroups,
+                     VT_KV_HEADS, full);
+        return;
+    }
+    if (vt_check(hipStreamSynchronize(g_vt.stream), "decode grid: sync")) return;
+    (void)vt_step_poll_abort();
+    if (vt_check(hipMemset(g_vt.d_bar_flags, 0, sizeof(unsigned) * VT_FLAG_COPIES * VT_FLAG_STRIDE), "decode grid: flags")) return;
+    g_vt.bar_epoch = 0;
+    g_vt.grid = grid;
+}
+
 /* Called by every entry point right after it has synchronised with the library's stream: if a
  * whole-step kernel ran since the last look, reads its abort flag (a 4-byte copy) and reports a
  * timed-out barrier like any other failed call.  Returns -1 if a step had been abandoned. */
