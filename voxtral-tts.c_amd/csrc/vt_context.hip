@@ -194,7 +194,7 @@ static void teardown(void) {
                     g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu,
                     g_vt.d_rope, g_vt.d_x, g_vt.d_q, g_vt.d_attn, g_vt.d_h, g_vt.d_att_part,
                     g_vt.d_att_cnt, g_vt.d_embed, g_vt.d_hidden, g_vt.d_bar_flags,
-                    g_vt.d_abort, g_vt.d_dummy, g_vt.d_scratch};
+                    g_vt.d_abort, g_vt.d_dummy, g_vt.d_scratch, g_vt.d_kv_img};
     for (size_t i = 0; i < sizeof ptrs / sizeof ptrs[0]; i++)
         if (ptrs[i]) (void)hipFree(ptrs[i]);
     if (g_vt.h_pin) (void)hipHostFree(g_vt.h_pin);

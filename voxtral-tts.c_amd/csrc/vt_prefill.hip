@@ -15,53 +15,18 @@
 #include <math.h>
 
 
-/* ---- RoPE + cache append ------------------------------------------------------- */
-
-/* qkv [S,6144] (the sum of `planes` split-K planes, `plane_stride` floats apart) ->
- * q [S,4096] with RoPE, cache rows start_pos.. (k with RoPE, v); only the columns from col0 on (a
- * multiple of 4; VT_Q_DIM: the cache rows alone, for an attention that takes q from the planes itself) */
-__global__ void vt_split_qkv_rope_kernel(const float *qkv, int planes, size_t plane_stride, float *q,
-                                         float *kc, float *vc, const float *rope, int start_pos, int S, int col0) {
-    /* a thread owns two adjacent RoPE pairs: 16-byte loads and stores */
-    const int quads = (VT_QKV_DIM - col0) / 4;
-    const size_t total = (size_t)S * quads;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-         i += (size_t)gridDim.x * blockDim.x) {
-        const int s = (int)(i / quads), g = col0 + (int)(i % quads) * 4;
-        f32x4 ab = *reinterpret_cast<const f32x4 *>(qkv + (size_t)s * VT_QKV_DIM + g);
-        for (int p = 1; p < planes; p++) {
-            const f32x4 w = *reinterpret_cast<const f32x4 *>(qkv + p * plane_stride + (size_t)s * VT_QKV_DIM + g);
-            ab.x = __fadd_rn(ab.x, w.x); ab.y = __fadd_rn(ab.y, w.y);
-            ab.z = __fadd_rn(ab.z, w.z); ab.w = __fadd_rn(ab.w, w.w);
-        }
-        f32x4 o = ab;
-        float *dst;
-        if (g < VT_Q_DIM + VT_KV_DIM) {
-            const int d = (g & (VT_HEAD_DIM - 1)) >> 1;         /* first of the two pairs */
-            const f32x4 cs = *reinterpret_cast<const f32x4 *>(rope + (size_t)(start_pos + s) * VT_HEAD_DIM + 2 * d);
-            o.x = __fsub_rn(__fmul_rn(ab.x, cs.x), __fmul_rn(ab.y, cs.y));
-            o.y = __fadd_rn(__fmul_rn(ab.x, cs.y), __fmul_rn(ab.y, cs.x));
-            o.z = __fsub_rn(__fmul_rn(ab.z, cs.z), __fmul_rn(ab.w, cs.w));
-            o.w = __fadd_rn(__fmul_rn(ab.z, cs.w), __fmul_rn(ab.w, cs.z));
-            dst = g < VT_Q_DIM ? q + (size_t)s * VT_Q_DIM + g
-                               : kc + (size_t)(start_pos + s) * VT_KV_DIM + (g - VT_Q_DIM);
-        } else {
-            dst = vc + (size_t)(start_pos + s) * VT_KV_DIM + (g - VT_Q_DIM - VT_KV_DIM);
-        }
-        *reinterpret_cast<f32x4 *>(dst) = o;
-    }
-}
-
 /* ---- causal attention, 16 queries x 32 keys per matrix-core tile ----------------
  * (tts_causal_attention, voxtral_tts_kernels.c:403-465, for head_dim 128 and four
  * query heads per KV head.)
  *
  * Workgroup = (KV head, HPW of its 4 query heads, block of 16 queries), HPW*NSPLIT
  * waves: wave = (query head, key-tile residue).  The waves of one residue share 32-key
- * K and V tiles in LDS, converted to (hi, lo) planes once, by the threads that fetched them, and
- * laid out as the matrix instructions want them: K as [key][dim] (a lane's operand is 8 consecutive
- * dims of a key), V transposed as [dim][lane group][8 key slots] (a lane's operand is the 8 keys of
- * its group for one dim).  Both products run on the bf16 matrix cores
+ * K and V tiles in LDS, as (hi, lo) planes laid out as the matrix instructions want them: K as
+ * [key][dim] (a lane's operand is 8 consecutive dims of a key), V transposed as [dim][lane
+ * group][8 key slots] (a lane's operand is the 8 keys of its group for one dim).  The planes are
+ * made once per layer, by vt_kv_image_kernel, in exactly this layout; a workgroup copies a tile's
+ * 38 KB image into its LDS (converting in here cost every step 1450 of its 5900 cycles, and every
+ * tile is used by 34 workgroups on average).  Both products run on the bf16 matrix cores
  * (v_mfma_f32_16x16x32_bf16) with every fp32 operand split in (hi, lo) bf16 planes as in
  * the projections: a b = hi_a hi_b + hi_a lo_b + lo_a hi_b, 16 mantissa bits per operand,
  * fp32 accumulation; three such instructions take 3/16 of the time of the fp32 ones they
@@ -78,9 +43,9 @@ __global__ void vt_split_qkv_rope_kernel(const float *qkv, int planes, size_t pl
 #define PA_QT 16                  /* queries per workgroup */
 #define PA_KROW 272               /* bytes per key of a K plane: 128 bf16 + 16 (16-byte reads over 16 keys cover all banks) */
 #define PA_VROW 80                /* bytes per dim of a V plane: 4 lane groups x 8 key slots + 16 */
-/* Dim d of V sits in row (d % 4) * 34 + d / 4 of its plane: a staging thread writes the same key slots of 4
- * consecutive dims, and a wave of them dims 4 apart, which in dim order would be rows 320 bytes apart, two
- * bank groups for eight lanes.  This way the lanes of a 16-byte write are consecutive rows, and the eight
+/* Dim d of V sits in row (d % 4) * 34 + d / 4 of its plane: a thread of the image kernel writes the same key
+ * slots of 4 consecutive dims, and a wave of them dims 4 apart, which in dim order would be rows 320 bytes
+ * apart.  This way the lanes of a 16-byte write are consecutive rows, and the eight
  * lanes of a 16-byte read (dims li = 0 .. 7 of a block: rows (li % 4) * 34 + li / 4) still cover all banks,
  * because 34 * 80 bytes is 2 of the 8 bank groups further on. */
 #define PA_VSKEW 34
@@ -101,15 +66,114 @@ __device__ __forceinline__ void pa_planes8(const f32x4 &a, const f32x4 &b, bf16x
     lo = __builtin_bit_cast(bf16x8, u32x4{l0, l1, l2, l3});
 }
 
+/* K and V of one layer as the attention wants them in its LDS: per (kv head, tile of 32 keys) the image
+ * [K hi plane | K lo plane | V hi plane | V lo plane] described above, img[kvh][tile], so that the attention
+ * copies a tile instead of converting it (every tile is read by all later query blocks of 4 heads: at 512
+ * rows 34 times on average).  Workgroup = (tile, kv head), 128 threads for K and 128 for V; thread (sg, cg) owns the dims
+ * 4*cg .. + 4 of the 8 keys that lane group sg meets in the second product (slot j: key 16*(j/4) + 4*sg +
+ * j%4), so that the transposed V write is one 16-byte store per dim and plane.
+ * Rows [start_pos, start_pos + S) come from the q|k|v product when qkv != NULL: the sum of `planes`
+ * split-K planes (`plane_stride` floats apart, fixed order), k rotated (adjacent pairs,
+ * voxtral_tts_kernels.c:616-634; the table holds (cos, sin) per pair), and are appended to the cache on the
+ * way (voxtral_tts_llm.c:317-324).  Earlier rows come from the cache; rows from kv_rows on are zeros (their
+ * keys are masked).  qkv == NULL: all rows are in the cache (rope is not read). */
+__global__ void __launch_bounds__(256)
+vt_kv_image_kernel(unsigned char *img, int img_tiles, const float *qkv, int planes, size_t plane_stride,
+                   float *kc, float *vc, const float *rope, int start_pos, int kv_rows) {
+    /* threads 0..127 make the K planes of the tile, threads 128..255 the V planes */
+    const int tile = (int)blockIdx.x, kvh = (int)blockIdx.y;
+    const bool is_v = threadIdx.x >= 128;
+    const int tl = (int)threadIdx.x & 127, sg = tl >> 5, cg = tl & 31;
+    const int col = kvh * VT_HEAD_DIM + 4 * cg;
+    float *cache = is_v ? vc : kc;
+    f32x4 r8[8];
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    if (qkv && tile * 32 >= start_pos && tile * 32 + 32 <= kv_rows) {
+        /* a tile of new rows only (all but the first and the last one of a chunk): every request up front */
+        const float *src = qkv + (size_t)(tile * 32 - start_pos) * VT_QKV_DIM + VT_Q_DIM + (is_v ? VT_KV_DIM : 0) + col;
+        f32x4 cs[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int row = 16 * (i >> 2) + 4 * sg + (i & 3);
+            r8[i] = *reinterpret_cast<const f32x4 *>(src + (size_t)row * VT_QKV_DIM);
+            cs[i] = is_v ? zero : *reinterpret_cast<const f32x4 *>(rope + (size_t)(tile * 32 + row) * VT_HEAD_DIM + 4 * cg);
+        }
+        for (int p = 1; p < planes; p++) {
+            f32x4 w[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                w[i] = *reinterpret_cast<const f32x4 *>(src + p * plane_stride + (size_t)(16 * (i >> 2) + 4 * sg + (i & 3)) * VT_QKV_DIM);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                r8[i].x = __fadd_rn(r8[i].x, w[i].x); r8[i].y = __fadd_rn(r8[i].y, w[i].y);
+                r8[i].z = __fadd_rn(r8[i].z, w[i].z); r8[i].w = __fadd_rn(r8[i].w, w[i].w);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int r = tile * 32 + 16 * (i >> 2) + 4 * sg + (i & 3);
+            if (!is_v) {
+                const f32x4 k = r8[i], c = cs[i];
+                r8[i] = f32x4{__fsub_rn(__fmul_rn(k.x, c.x), __fmul_rn(k.y, c.y)), __fadd_rn(__fmul_rn(k.x, c.y), __fmul_rn(k.y, c.x)),
+                              __fsub_rn(__fmul_rn(k.z, c.z), __fmul_rn(k.w, c.w)), __fadd_rn(__fmul_rn(k.z, c.w), __fmul_rn(k.w, c.z))};
+            }
+            *reinterpret_cast<f32x4 *>(cache + (size_t)r * VT_KV_DIM + col) = r8[i];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int r = tile * 32 + 16 * (i >> 2) + 4 * sg + (i & 3);
+            if (r >= kv_rows) {
+                r8[i] = zero;
+            } else if (qkv && r >= start_pos) {
+                const float *src = qkv + (size_t)(r - start_pos) * VT_QKV_DIM + VT_Q_DIM + (is_v ? VT_KV_DIM : 0) + col;
+                f32x4 k = *reinterpret_cast<const f32x4 *>(src);
+                for (int p = 1; p < planes; p++) {
+                    const f32x4 k2 = *reinterpret_cast<const f32x4 *>(src + p * plane_stride);
+                    k.x = __fadd_rn(k.x, k2.x); k.y = __fadd_rn(k.y, k2.y); k.z = __fadd_rn(k.z, k2.z); k.w = __fadd_rn(k.w, k2.w);
+                }
+                if (!is_v) {
+                    const f32x4 c = *reinterpret_cast<const f32x4 *>(rope + (size_t)r * VT_HEAD_DIM + 4 * cg);
+                    k = f32x4{__fsub_rn(__fmul_rn(k.x, c.x), __fmul_rn(k.y, c.y)), __fadd_rn(__fmul_rn(k.x, c.y), __fmul_rn(k.y, c.x)),
+                              __fsub_rn(__fmul_rn(k.z, c.z), __fmul_rn(k.w, c.w)), __fadd_rn(__fmul_rn(k.z, c.w), __fmul_rn(k.w, c.z))};
+                }
+                *reinterpret_cast<f32x4 *>(cache + (size_t)r * VT_KV_DIM + col) = k;
+                r8[i] = k;
+            } else {
+                r8[i] = *reinterpret_cast<const f32x4 *>(cache + (size_t)r * VT_KV_DIM + col);
+            }
+        }
+    }
+    unsigned char *Kt = img + ((size_t)kvh * img_tiles + tile) * PA_TILE_BYTES, *Vt = Kt + 2 * PA_KPLANE;
+    if (!is_v) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int row = 16 * (i >> 2) + 4 * sg + (i & 3);
+            u32x2 h, l;
+            vt_split_planes4(r8[i].x, r8[i].y, r8[i].z, r8[i].w, h, l);
+            *reinterpret_cast<u32x2 *>(Kt + row * PA_KROW + 8 * cg) = h;
+            *reinterpret_cast<u32x2 *>(Kt + PA_KPLANE + row * PA_KROW + 8 * cg) = l;
+        }
+    } else {
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            bf16x8 h, l;
+            pa_planes8(f32x4{r8[0][d], r8[1][d], r8[2][d], r8[3][d]}, f32x4{r8[4][d], r8[5][d], r8[6][d], r8[7][d]}, h, l);
+            *reinterpret_cast<bf16x8 *>(Vt + (d * PA_VSKEW + cg) * PA_VROW + 16 * sg) = h;
+            *reinterpret_cast<bf16x8 *>(Vt + PA_VPLANE + (d * PA_VSKEW + cg) * PA_VROW + 16 * sg) = l;
+        }
+    }
+}
+
 template <int NSPLIT, int HPW>
 __global__ void __launch_bounds__(64 * HPW * NSPLIT)
 vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, const float *Q,
                             int q_stride, int q_planes, size_t q_plane_stride, const float *rope,
-                            const float *Kc, const float *Vc, int S, int start_pos, float scale) {
+                            const unsigned char *img, int img_tiles, int S, int start_pos, float scale) {
     extern __shared__ __attribute__((aligned(16))) unsigned char pa_lds[];
     constexpr int GT = 64 * HPW;                         /* threads of a residue group */
-    constexpr int NLD = 1024 / GT;                       /* 16-byte loads per thread and tile */
-    static_assert(GT == 128, "a staging thread owns the 8 key slots of one lane group");
+    constexpr int NCH = PA_TILE_BYTES / 16;              /* 16-byte chunks of a tile image */
+    constexpr int NLD = (NCH + GT - 1) / GT;             /* chunks per thread and tile */
     const int kvh = (int)blockIdx.x / (4 / HPW), hsub = (int)blockIdx.x % (4 / HPW);
     /* The last query block has the most keys.  Workgroups are handed to the CUs in launch order, one per
      * CU and then a second one each: the first half of the launch takes the long blocks in descending
@@ -126,53 +190,54 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
     const int head = kvh * 4 + hsub * HPW + hq;
     unsigned char *Kt = pa_lds + (size_t)pz * PA_TILE_BYTES, *Vt = Kt + 2 * PA_KPLANE;   /* hi plane, then lo */
 
-    /* The workgroups of one blockIdx.x run on one XCD and walk the same K and V rows, tile by tile, at the
-     * same pace: left alone, every tile is a miss in that XCD's L2 for all of them at the moment they need
-     * it, and each step pays the full memory latency.  So they first touch all the rows between them, one
-     * 128-byte line per lane and request (K and V rows are 4 lines each), which starts every line on its way
-     * into the L2 at once.  The values are dropped at the end of the kernel. */
-    unsigned warm[4];
-    {
-        const int n_lines = (start_pos + S) * 8, stride = (int)(gridDim.y * blockDim.x);
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            int j = (int)blockIdx.y * (int)blockDim.x + t + k * stride;
-            j = j < n_lines ? j : n_lines - 1;
-            const int which = j & 1, row = j >> 3, line = (j >> 1) & 3;
-            warm[k] = *reinterpret_cast<const unsigned *>((which ? Vc : Kc) + (size_t)row * VT_KV_DIM + kvh * VT_HEAD_DIM + line * 32);
-        }
-    }
-
     /* this lane's query as the B operand of K Q^T: dims 8*g + 32*ks .. + 8 for K step ks, both planes */
     bf16x8 qhi[4], qlo[4];
     {
         /* Q as it is, or (rope != NULL) the raw product: the sum of q_planes split-K planes, rotated here
-         * (adjacent pairs, voxtral_tts_kernels.c:616-634; the table holds (cos, sin) per pair) */
+         * (adjacent pairs, voxtral_tts_kernels.c:616-634; the table holds (cos, sin) per pair).  All
+         * requests of a plane go out before the first value is used: inside a prefill every one of them
+         * goes to memory, and one after the other they were 7 us of a 27 us launch. */
         const int qrow = my_q < S ? my_q : S - 1;
         const float *qp = Q + (size_t)qrow * q_stride + head * VT_HEAD_DIM + 8 * g;
-        const float *cs = rope ? rope + (size_t)(start_pos + qrow) * VT_HEAD_DIM + 8 * g : NULL;
+        f32x4 qa[4], qb[4];
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            f32x4 a = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[0];
-            f32x4 b = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[1];
-            if (rope) {
-                for (int p = 1; p < q_planes; p++) {
-                    const f32x4 a2 = reinterpret_cast<const f32x4 *>(qp + p * q_plane_stride + 32 * ks)[0];
-                    const f32x4 b2 = reinterpret_cast<const f32x4 *>(qp + p * q_plane_stride + 32 * ks)[1];
-                    a.x = __fadd_rn(a.x, a2.x); a.y = __fadd_rn(a.y, a2.y); a.z = __fadd_rn(a.z, a2.z); a.w = __fadd_rn(a.w, a2.w);
-                    b.x = __fadd_rn(b.x, b2.x); b.y = __fadd_rn(b.y, b2.y); b.z = __fadd_rn(b.z, b2.z); b.w = __fadd_rn(b.w, b2.w);
-                }
-                const f32x4 c0 = reinterpret_cast<const f32x4 *>(cs + 32 * ks)[0];
-                const f32x4 c1 = reinterpret_cast<const f32x4 *>(cs + 32 * ks)[1];
-                const f32x4 ra = {__fsub_rn(__fmul_rn(a.x, c0.x), __fmul_rn(a.y, c0.y)), __fadd_rn(__fmul_rn(a.x, c0.y), __fmul_rn(a.y, c0.x)),
-                                  __fsub_rn(__fmul_rn(a.z, c0.z), __fmul_rn(a.w, c0.w)), __fadd_rn(__fmul_rn(a.z, c0.w), __fmul_rn(a.w, c0.z))};
-                const f32x4 rb = {__fsub_rn(__fmul_rn(b.x, c1.x), __fmul_rn(b.y, c1.y)), __fadd_rn(__fmul_rn(b.x, c1.y), __fmul_rn(b.y, c1.x)),
-                                  __fsub_rn(__fmul_rn(b.z, c1.z), __fmul_rn(b.w, c1.w)), __fadd_rn(__fmul_rn(b.z, c1.w), __fmul_rn(b.w, c1.z))};
-                a = ra;
-                b = rb;
-            }
-            pa_planes8(a, b, qhi[ks], qlo[ks]);
+            qa[ks] = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[0];
+            qb[ks] = reinterpret_cast<const f32x4 *>(qp + 32 * ks)[1];
         }
+        if (rope) {
+            const float *cs = rope + (size_t)(start_pos + qrow) * VT_HEAD_DIM + 8 * g;
+            f32x4 c0[4], c1[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                c0[ks] = reinterpret_cast<const f32x4 *>(cs + 32 * ks)[0];
+                c1[ks] = reinterpret_cast<const f32x4 *>(cs + 32 * ks)[1];
+            }
+            for (int p = 1; p < q_planes; p++) {
+                f32x4 a2[4], b2[4];
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) {
+                    a2[ks] = reinterpret_cast<const f32x4 *>(qp + p * q_plane_stride + 32 * ks)[0];
+                    b2[ks] = reinterpret_cast<const f32x4 *>(qp + p * q_plane_stride + 32 * ks)[1];
+                }
+#pragma unroll
+                for (int ks = 0; ks < 4; ks++) {
+                    f32x4 &a = qa[ks], &b = qb[ks];
+                    a.x = __fadd_rn(a.x, a2[ks].x); a.y = __fadd_rn(a.y, a2[ks].y); a.z = __fadd_rn(a.z, a2[ks].z); a.w = __fadd_rn(a.w, a2[ks].w);
+                    b.x = __fadd_rn(b.x, b2[ks].x); b.y = __fadd_rn(b.y, b2[ks].y); b.z = __fadd_rn(b.z, b2[ks].z); b.w = __fadd_rn(b.w, b2[ks].w);
+                }
+            }
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                const f32x4 a = qa[ks], b = qb[ks];
+                qa[ks] = f32x4{__fsub_rn(__fmul_rn(a.x, c0[ks].x), __fmul_rn(a.y, c0[ks].y)), __fadd_rn(__fmul_rn(a.x, c0[ks].y), __fmul_rn(a.y, c0[ks].x)),
+                               __fsub_rn(__fmul_rn(a.z, c0[ks].z), __fmul_rn(a.w, c0[ks].w)), __fadd_rn(__fmul_rn(a.z, c0[ks].w), __fmul_rn(a.w, c0[ks].z))};
+                qb[ks] = f32x4{__fsub_rn(__fmul_rn(b.x, c1[ks].x), __fmul_rn(b.y, c1[ks].y)), __fadd_rn(__fmul_rn(b.x, c1[ks].y), __fmul_rn(b.y, c1[ks].x)),
+                               __fsub_rn(__fmul_rn(b.z, c1[ks].z), __fmul_rn(b.w, c1[ks].w)), __fadd_rn(__fmul_rn(b.z, c1[ks].w), __fmul_rn(b.w, c1[ks].z))};
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) pa_planes8(qa[ks], qb[ks], qhi[ks], qlo[ks]);
     }
     f32x4 o[8];
 #pragma unroll
@@ -182,30 +247,29 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
     const int last_q = (q0 + PA_QT - 1 < S ? q0 + PA_QT - 1 : S - 1) + start_pos;
     const int ntiles = last_q / 32 + 1;                  /* key tiles 0 .. ntiles-1 are visible */
     const int nsteps = (ntiles + NSPLIT - 1) / NSPLIT;
-    const int kv_rows = start_pos + S;
 
-    /* staging: the threads of a residue group move 32 rows x 512 B of K and of V.  Thread (sg, cg) takes
-     * the 4 dims 4*cg .. of the 8 keys that lane group sg meets in the second product (slot j: key
-     * 16*(j/4) + 4*sg + j%4). */
-    const int sg = tl >> 5, cg = tl & 31;
-    f32x4 rk[NLD], rv[NLD];
-    /* buffer loads: the tile's first row as the scalar offset, this thread's row and columns as a vector
-     * offset that never changes (no 64-bit address arithmetic per load), and rows past the end of the
-     * cache read as zeros (their keys are masked) */
-    const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc((void *)(Kc + kvh * VT_HEAD_DIM), 0,
-                                                                          kv_rows * VT_KV_DIM * 4 - kvh * VT_HEAD_DIM * 4, 0x00020000);
-    const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc((void *)(Vc + kvh * VT_HEAD_DIM), 0,
-                                                                          kv_rows * VT_KV_DIM * 4 - kvh * VT_HEAD_DIM * 4, 0x00020000);
+    /* staging: a tile arrives as the image vt_kv_image_kernel made of it, which is what the LDS holds:
+     * the threads of a residue group copy its 16-byte chunks tl, tl + GT, ...  Buffer loads: the tile as the
+     * scalar offset, the thread's chunk as a vector offset that never changes (no 64-bit address arithmetic
+     * per load); the chunks past the end of a tile belong to nobody and are never stored. */
+    u32x4 rt[NLD];
+    const __amdgpu_buffer_rsrc_t t_rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(img + (size_t)kvh * img_tiles * PA_TILE_BYTES), 0, img_tiles * PA_TILE_BYTES, 0x00020000);
     int voff[NLD];
 #pragma unroll
-    for (int i = 0; i < NLD; i++) voff[i] = (16 * (i >> 2) + 4 * sg + (i & 3)) * (VT_KV_DIM * 4) + 16 * cg;
-    auto fetch = [&](int tile) {
-        const int soff = __builtin_amdgcn_readfirstlane(tile) * (32 * VT_KV_DIM * 4);
+    for (int i = 0; i < NLD; i++) voff[i] = 16 * (tl + GT * i < NCH ? tl + GT * i : NCH - 1);
+    /* A tile is requested in four parts, dealt out over the step: a wave's requests are accepted at the
+     * pace at which the CU's address unit works them off (16 cycles per 1 KB request, all waves of the CU
+     * together), and all of them in a row hold the wave's own matrix instructions up behind them. */
+    auto fetch_part = [&](int tile, int part) {
+        const int soff = __builtin_amdgcn_readfirstlane(tile) * PA_TILE_BYTES;
 #pragma unroll
-        for (int i = 0; i < NLD; i++) {
-            rk[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(k_rs, voff[i], soff, 0));
-            rv[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(v_rs, voff[i], soff, 0));
-        }
+        for (int i = (part * NLD) / 4; i < ((part + 1) * NLD) / 4; i++)
+            rt[i] = __builtin_amdgcn_raw_buffer_load_b128(t_rs, voff[i], soff, 0);
+    };
+    auto fetch = [&](int tile) {
+#pragma unroll
+        for (int part = 0; part < 4; part++) fetch_part(tile, part);
     };
     /* Every request of the loop below is unconditional (a tile index beyond the last visible one
      * is clamped: that tile is fetched again, out of the L2, and never stored): behind a
@@ -213,31 +277,40 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
      * anything loaded, here the query registers, i.e. before the products of every step. */
     fetch(pz < ntiles ? pz : ntiles - 1);
 
+    /* The workgroups of one blockIdx.x run on one XCD and walk the same K and V rows, tile by tile, at the
+     * same pace: left alone, every tile is a miss in that XCD's L2 for all of them at the moment they need
+     * it, and each step pays the full memory latency.  So they first touch all the rows between them, one
+     * 128-byte line per lane and request (K and V rows are 4 lines each), which starts every line on its way
+     * into the L2 at once.  The values are dropped at the end of the kernel. */
+    unsigned warm[4];
+    {   /* (behind the query and the first tile: a wave's loads return in order, and these go all the way to memory) */
+        const int n_lines = ((start_pos + S + 31) / 32) * (PA_TILE_BYTES / 128), stride = (int)(gridDim.y * blockDim.x);
+        const unsigned char *mine = img + (size_t)kvh * img_tiles * PA_TILE_BYTES;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            int j = (int)blockIdx.y * (int)blockDim.x + t + k * stride;
+            j = j < n_lines ? j : n_lines - 1;
+            warm[k] = *reinterpret_cast<const unsigned *>(mine + (size_t)j * 128);
+        }
+    }
+
     for (int step = 0; step < nsteps; step++) {
         const int tile = step * NSPLIT + pz;
         const bool valid = tile < ntiles;
         __syncthreads();
         if (valid) {
 #pragma unroll
-            for (int i = 0; i < NLD; i++) {
-                const int row = 16 * (i >> 2) + 4 * sg + (i & 3);
-                u32x2 h, l;
-                vt_split_planes4(rk[i].x, rk[i].y, rk[i].z, rk[i].w, h, l);
-                *reinterpret_cast<u32x2 *>(Kt + row * PA_KROW + 8 * cg) = h;
-                *reinterpret_cast<u32x2 *>(Kt + PA_KPLANE + row * PA_KROW + 8 * cg) = l;
-            }
-#pragma unroll
-            for (int d = 0; d < 4; d++) {
-                bf16x8 h, l;
-                pa_planes8(f32x4{rv[0][d], rv[1][d], rv[2][d], rv[3][d]}, f32x4{rv[4][d], rv[5][d], rv[6][d], rv[7][d]}, h, l);
-                *reinterpret_cast<bf16x8 *>(Vt + (d * PA_VSKEW + cg) * PA_VROW + 16 * sg) = h;
-                *reinterpret_cast<bf16x8 *>(Vt + PA_VPLANE + (d * PA_VSKEW + cg) * PA_VROW + 16 * sg) = l;
-            }
+            for (int i = 0; i < NLD; i++)
+                if (GT * (i + 1) <= NCH || tl + GT * i < NCH) *reinterpret_cast<u32x4 *>(Kt + 16 * (tl + GT * i)) = rt[i];
         }
         __syncthreads();
-        fetch(tile + NSPLIT < ntiles ? tile + NSPLIT : ntiles - 1);
-        __builtin_amdgcn_sched_barrier(0);               /* requests first, products behind them */
-        if (!valid) continue;
+        const int nxt = tile + NSPLIT < ntiles ? tile + NSPLIT : ntiles - 1;
+        fetch_part(nxt, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (!valid) {
+            fetch_part(nxt, 1); fetch_part(nxt, 2); fetch_part(nxt, 3);
+            continue;
+        }
 
         /* S^T = K Q^T: K step ks pairs the dims 8*g + 32*ks .. + 8 of key 16*kb + li and of the query */
         f32x4 s[2];
@@ -254,6 +327,9 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
                 s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(khi, qhi[ks], s[kb], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_part(nxt, 1);
+        __builtin_amdgcn_sched_barrier(0);
         /* online softmax for this lane's query; element v of block kb is key 16*kb + 4*g + v */
         const int qpos = start_pos + my_q;
         float mx = -1e30f;
@@ -285,6 +361,9 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
          * s[j/4][j%4]; the A operand of dim block b is that key's column 16*b + li of V */
         bf16x8 phi, plo;
         pa_planes8(s[0], s[1], phi, plo);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_part(nxt, 2);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int b = 0; b < 8; b++) {
             const unsigned char *vp = Vt + ((li & 3) * PA_VSKEW + 4 * b + (li >> 2)) * PA_VROW + 16 * g;
@@ -294,6 +373,8 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
             o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vhi, plo, o[b], 0, 0, 0);
             o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vhi, phi, o[b], 0, 0, 0);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_part(nxt, 3);
     }
 
     /* merge the residues: residue r > 0 parks (m, l, O) in LDS, residue 0 folds them in */
@@ -361,12 +442,38 @@ static size_t pa_lds_bytes(void) {
     return tiles > park ? tiles : park;
 }
 
+/* Tiles of 32 keys that cover `rows` cache rows, and the tile images of one layer's K and V (a buffer of the
+ * library's own that grows with the longest cache seen) */
+static int pa_tiles(int rows) { return (rows + 31) / 32; }
+static unsigned char *pa_image(int rows) {
+    const size_t bytes = (size_t)VT_KV_HEADS * pa_tiles(rows) * PA_TILE_BYTES;
+    if (bytes > g_vt.kv_img_bytes) {
+        if (g_vt.d_kv_img) {
+            (void)hipStreamSynchronize(g_vt.stream);
+            (void)hipFree(g_vt.d_kv_img);
+        }
+        g_vt.d_kv_img = vt_dev_alloc(bytes);
+        g_vt.kv_img_bytes = g_vt.d_kv_img ? bytes : 0;
+    }
+    return (unsigned char *)g_vt.d_kv_img;
+}
+
+/* d_qkv != NULL: rows start_pos .. start_pos + S - 1 are taken from the q|k|v product (summed, k rotated)
+ * and appended to the cache d_K / d_V; otherwise all start_pos + S rows are in the cache already */
+static void pa_launch_image(unsigned char *d_img, const float *d_qkv, int planes, size_t plane_stride, float *d_K,
+                            float *d_V, int S, int start_pos) {
+    const int rows = start_pos + S;
+    hipLaunchKernelGGL(vt_kv_image_kernel, dim3(pa_tiles(rows), VT_KV_HEADS), dim3(256), 0, g_vt.stream, d_img,
+                       pa_tiles(rows), d_qkv, planes, plane_stride, d_K, d_V, g_vt.d_rope, start_pos, rows);
+}
+
 /* Q rows are q_stride floats apart; out / (out_hi, out_lo) are [S,4096], each optional.  d_rope != NULL: d_Q
  * holds q_planes split-K planes (q_plane_stride floats apart) of the raw q product, to be summed and
- * rotated with the table rows start_pos .. by the kernel. */
+ * rotated with the table rows start_pos .. by the kernel.  d_img: the tile images of the start_pos + S
+ * cache rows (vt_kv_image_kernel). */
 void vt_launch_prefill_attention_raw(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
                                      int q_stride, int q_planes, size_t q_plane_stride, const float *d_rope,
-                                     const float *d_K, const float *d_V, int S, int start_pos, float scale) {
+                                     const unsigned char *d_img, int S, int start_pos, float scale) {
     static int attr_set = 0;
     if (!attr_set) {
         if (vt_check(hipFuncSetAttribute((const void *)vt_prefill_attention_kernel<PA_NSPLIT, PA_HPW>,
@@ -378,13 +485,17 @@ void vt_launch_prefill_attention_raw(float *d_out, uint16_t *d_hi, uint16_t *d_l
     hipLaunchKernelGGL((vt_prefill_attention_kernel<PA_NSPLIT, PA_HPW>),
                        dim3(VT_KV_HEADS * (4 / PA_HPW), (S + PA_QT - 1) / PA_QT), dim3(64 * PA_HPW * PA_NSPLIT),
                        pa_lds_bytes(), g_vt.stream, d_out, d_hi, d_lo, d_Q, q_stride, q_planes, q_plane_stride, d_rope,
-                       d_K, d_V, S, start_pos, scale);
+                       d_img, pa_tiles(start_pos + S), S, start_pos, scale);
 }
 
 void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
                                  int q_stride, const float *d_K, const float *d_V, int S, int start_pos,
                                  float scale) {
-    vt_launch_prefill_attention_raw(d_out, d_hi, d_lo, d_Q, q_stride, 1, 0, NULL, d_K, d_V, S, start_pos, scale);
+    unsigned char *img = pa_image(start_pos + S);
+    if (!img) return;
+    /* (the image kernel only reads a cache that is complete) */
+    pa_launch_image(img, NULL, 0, 0, const_cast<float *>(d_K), const_cast<float *>(d_V), S, start_pos);
+    vt_launch_prefill_attention_raw(d_out, d_hi, d_lo, d_Q, q_stride, 1, 0, NULL, img, S, start_pos, scale);
 }
 
 /* ---- backbone prefill ------------------------------------------------------------ */
@@ -398,8 +509,6 @@ static int vt_prefill_cuts(int tiles, int most) {
     const int c = g_vt.n_cu / tiles;
     return c < 1 ? 1 : c > most ? most : c;
 }
-
-static int ew_blocks(size_t n) { size_t b = (n + 255) / 256; return (int)(b > 8192 ? 8192 : b); }
 
 extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int start_pos, float *out_x) {
     if (!g_vt.initialized || g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_llm_prefill: no weights uploaded"); return; }
@@ -419,12 +528,13 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
     /* the 128 x 128 kernel on row-major weights (layers without a fragment copy) wants cuts that divide K */
     const int rq = m_tiles >= 3 ? 2 : 4, ro = m_tiles >= 3 ? 4 : 8;
     const int tail_cols = m_tiles == 4 ? 16 * 128 : 0;      /* part holds 4 x S x 2048 <= 8 x S x 3072 */
-    const size_t n_x = S * VT_DIM, n_wide = S * 4 * VT_QKV_DIM, n_q = S * VT_Q_DIM, n_part = 8 * S * VT_DIM;
+    const size_t n_x = S * VT_DIM, n_wide = S * 4 * VT_QKV_DIM, n_part = 8 * S * VT_DIM;
     const size_t n_plane = S * VT_FFN;                            /* bf16 elements per plane */
-    const size_t bytes = sizeof(float) * (n_x + n_wide + n_q + n_part) + 2 * sizeof(uint16_t) * n_plane;
+    const size_t bytes = sizeof(float) * (n_x + n_wide + n_part) + 2 * sizeof(uint16_t) * n_plane;
     float *x = (float *)vt_scratch(bytes);
-    if (!x) return;
-    float *wide = x + n_x, *q = wide + n_wide, *part = q + n_q;
+    unsigned char *img = pa_image(start_pos + seq_len);
+    if (!x || !img) return;
+    float *wide = x + n_x, *part = wide + n_wide;
     uint16_t *hi = (uint16_t *)(part + n_part), *lo = hi + n_plane;
     const size_t ps = S * VT_DIM;
 
@@ -439,10 +549,10 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         const int sp_qkv = frag ? fq : rq, sp_wo = frag ? fo : ro, sp_w2 = sp_wo;
         if (frag) vt_launch_gemm_frag(wide, VT_QKV_DIM, S * VT_QKV_DIM, hi, lo, F->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
         else vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
-        /* k (rotated) and v into the cache; the attention takes q from the product's planes itself */
-        hipLaunchKernelGGL(vt_split_qkv_rope_kernel, dim3(ew_blocks(S * 2 * VT_KV_DIM / 4)), dim3(256), 0, st,
-                           wide, sp_qkv, S * VT_QKV_DIM, q, kc, vc, g_vt.d_rope, start_pos, seq_len, VT_Q_DIM);
-        vt_launch_prefill_attention_raw(NULL, hi, lo, wide, VT_QKV_DIM, sp_qkv, S * VT_QKV_DIM, g_vt.d_rope, kc, vc,
+        /* k (rotated) and v into the cache and, with the earlier rows, into the attention's tile images; the
+         * attention takes q from the product's planes itself */
+        pa_launch_image(img, wide, sp_qkv, S * VT_QKV_DIM, kc, vc, seq_len, start_pos);
+        vt_launch_prefill_attention_raw(NULL, hi, lo, wide, VT_QKV_DIM, sp_qkv, S * VT_QKV_DIM, g_vt.d_rope, img,
                                         seq_len, start_pos, VT_ATT_SCALE);
         if (frag) vt_launch_gemm_frag(part, VT_DIM, ps, hi, lo, F->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
         else vt_launch_gemm(part, hi, lo, L->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
@@ -522,6 +632,13 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
         vt_launch_bench_fill(hi, lo, n_plane);
     else                                              /* q: floats whose upper halves are such bf16 values */
         vt_launch_bench_fill((uint16_t *)q, NULL, 2 * n_q);
+    /* the attention alone: the tile images of layer 0's cache are made once, in front of the loop (in a
+     * prefill the kernel that appends the new rows to the cache writes them) */
+    unsigned char *img = NULL;
+    if (which == 4) {
+        if (!(img = pa_image(S))) return -1.f;
+        pa_launch_image(img, NULL, 0, 0, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu, S, 0);
+    }
     float ms = -1.f;
     for (int it = -2; it < iters; it++) {
         if (it == 0 && vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench start")) return -1.f;
@@ -544,7 +661,7 @@ extern "C" float tts_hip_bench_kernel(int which, int iters) {
                               W[2] + (size_t)main_cols * VT_DIM, S, tail, VT_DIM, 4);
         } else if (which < 4 && frag) vt_launch_gemm_frag(out, NN[which], (size_t)S * NN[which], hi, lo, Wf[which], S, NN[which], KK[which], SP[which]);
         else if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], RP[which]);
-        else vt_launch_prefill_attention(out, NULL, NULL, q, VT_Q_DIM, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu, S, 0, VT_ATT_SCALE);
+        else vt_launch_prefill_attention_raw(out, NULL, NULL, q, VT_Q_DIM, 1, 0, NULL, img, S, 0, VT_ATT_SCALE);
     }
     if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;
     if (vt_check(hipEventSynchronize(g_vt.ev1), "bench sync")) return -1.f;

@@ -81,6 +81,8 @@ struct vt_state {
     /* generic scratch (prefill / acoustic / linear) */
     void *d_scratch;
     size_t scratch_bytes;
+    void *d_kv_img;               /* prefill attention: tile images of one layer's K and V */
+    size_t kv_img_bytes;
 
     int error_count;
     char last_error[512];
