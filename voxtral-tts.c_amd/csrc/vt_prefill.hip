@@ -25,7 +25,7 @@
  * [key][dim] (a lane's operand is 8 consecutive dims of a key), V transposed as [dim][lane
  * group][8 key slots] (a lane's operand is the 8 keys of its group for one dim).  The planes are
  * made once per layer, by vt_kv_image_kernel, in exactly this layout; a workgroup copies a tile's
- * 38 KB image into its LDS (converting in here cost every step 1450 of its 5900 cycles, and every
+ * 37 KB image into its LDS (converting in here cost every step 1450 of its 5900 cycles, and every
  * tile is used by 34 workgroups on average).  Both products run on the bf16 matrix cores
  * (v_mfma_f32_16x16x32_bf16) with every fp32 operand split in (hi, lo) bf16 planes as in
  * the projections: a b = hi_a hi_b + hi_a lo_b + lo_a hi_b, 16 mantissa bits per operand,
@@ -43,14 +43,11 @@
 #define PA_QT 16                  /* queries per workgroup */
 #define PA_KROW 272               /* bytes per key of a K plane: 128 bf16 + 16 (16-byte reads over 16 keys cover all banks) */
 #define PA_VROW 80                /* bytes per dim of a V plane: 4 lane groups x 8 key slots + 16 */
-/* Dim d of V sits in row (d % 4) * 34 + d / 4 of its plane: a thread of the image kernel writes the same key
- * slots of 4 consecutive dims, and a wave of them dims 4 apart, which in dim order would be rows 320 bytes
- * apart.  This way the lanes of a 16-byte write are consecutive rows, and the eight
- * lanes of a 16-byte read (dims li = 0 .. 7 of a block: rows (li % 4) * 34 + li / 4) still cover all banks,
- * because 34 * 80 bytes is 2 of the 8 bank groups further on. */
-#define PA_VSKEW 34
+/* Dim d of V is row d of its plane: the 16 lanes that a 16-byte LDS read serves together (dims 16 b + li of
+ * a block) then start 20 li dwords apart, which are 16 different groups of four banks.  (While the tiles were
+ * converted in here the rows were skewed to keep the transposed writes free of bank conflicts.) */
 #define PA_KPLANE (32 * PA_KROW)
-#define PA_VPLANE ((3 * PA_VSKEW + VT_HEAD_DIM / 4) * PA_VROW)
+#define PA_VPLANE (VT_HEAD_DIM * PA_VROW)
 #define PA_TILE_BYTES (2 * PA_KPLANE + 2 * PA_VPLANE)
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -159,8 +156,8 @@ vt_kv_image_kernel(unsigned char *img, int img_tiles, const float *qkv, int plan
         for (int d = 0; d < 4; d++) {
             bf16x8 h, l;
             pa_planes8(f32x4{r8[0][d], r8[1][d], r8[2][d], r8[3][d]}, f32x4{r8[4][d], r8[5][d], r8[6][d], r8[7][d]}, h, l);
-            *reinterpret_cast<bf16x8 *>(Vt + (d * PA_VSKEW + cg) * PA_VROW + 16 * sg) = h;
-            *reinterpret_cast<bf16x8 *>(Vt + PA_VPLANE + (d * PA_VSKEW + cg) * PA_VROW + 16 * sg) = l;
+            *reinterpret_cast<bf16x8 *>(Vt + (4 * cg + d) * PA_VROW + 16 * sg) = h;
+            *reinterpret_cast<bf16x8 *>(Vt + PA_VPLANE + (4 * cg + d) * PA_VROW + 16 * sg) = l;
         }
     }
 }
@@ -366,7 +363,7 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int b = 0; b < 8; b++) {
-            const unsigned char *vp = Vt + ((li & 3) * PA_VSKEW + 4 * b + (li >> 2)) * PA_VROW + 16 * g;
+            const unsigned char *vp = Vt + (16 * b + li) * PA_VROW + 16 * g;
             const bf16x8 vhi = *reinterpret_cast<const bf16x8 *>(vp);
             const bf16x8 vlo = *reinterpret_cast<const bf16x8 *>(vp + PA_VPLANE);
             o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vlo, phi, o[b], 0, 0, 0);
