@@ -151,7 +151,10 @@ void tts_hip_causal_attention_decode(float *d_out, const float *d_Q, const float
                                      const float *d_V_cache, int seq_k, int n_heads,
                                      int n_kv_heads, int head_dim, float scale,
                                      int kv_cache_stride);
-/* replaces tts_cuda_causal_attention_prefill (voxtral_tts_cuda.h:142-145) */
+/* replaces tts_cuda_causal_attention_prefill (voxtral_tts_cuda.h:142-145).  With the model's head
+ * counts and 8 or more queries it runs on the matrix cores, from tile images of K and V that a first
+ * kernel writes into a buffer of the library's own (8 x ceil((start_pos + seq_len) / 32) x 37 KB,
+ * allocated when a call needs more than any before it). */
 void tts_hip_causal_attention_prefill(float *d_out, const float *d_Q, const float *d_K,
                                       const float *d_V, int seq_len, int start_pos,
                                       int n_heads, int n_kv_heads, int head_dim, float scale);
