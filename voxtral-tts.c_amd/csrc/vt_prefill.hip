@@ -431,7 +431,9 @@ vt_prefill_attention_kernel(float *out, uint16_t *out_hi, uint16_t *out_lo, cons
 #ifndef PA_NSPLIT
 #define PA_NSPLIT 2
 #endif
+#ifndef PA_HPW
 #define PA_HPW 2
+#endif
 
 static size_t pa_lds_bytes(void) {
     size_t tiles = (size_t)PA_NSPLIT * PA_TILE_BYTES;
