@@ -78,8 +78,9 @@ def test_linear_closed_forms(hip):
     assert np.max(np.abs(y - want)) < 1e-4 * np.sqrt(k)
 
 
-@pytest.mark.parametrize("seq,start", [(512, 0), (77, 19), (32, 0), (33, 31), (8, 0)])
+@pytest.mark.parametrize("seq,start", [(8, 0), (77, 19), (512, 0), (32, 0), (33, 31)])
 def test_causal_attention_tiles(hip, orc, seq, start):
+    """(In this order the library's buffer of K/V tile images grows twice after it has been used.)"""
     Q = S.f32_normal((seq, S.Q_DIM), 700 + seq)
     K = S.f32_normal((start + seq, S.KV_DIM), 701 + seq)
     V = S.f32_normal((start + seq, S.KV_DIM), 702 + seq)
