@@ -24,11 +24,53 @@ from concurrent.futures import ThreadPoolExecutor
 import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-sys.path.insert(0, os.path.join(ROOT, "tests"))
-sys.path.insert(0, os.path.join(ROOT, "tests", "golden"))
 
-import hipsupport as H  # noqa: E402
-import vtsupport as S  # noqa: E402
+
+def _package():
+    """The package directory (its name is not a Python identifier): the ctypes mirror of the C ABI,
+    the seeded synthetic weights and the device session."""
+    import importlib.util
+    name = "voxtral_tts_c_amd"
+    if name not in sys.modules:
+        pkg_dir = os.path.join(ROOT, "voxtral-tts.c_amd")
+        spec = importlib.util.spec_from_file_location(name, os.path.join(pkg_dir, "__init__.py"),
+                                                      submodule_search_locations=[pkg_dir])
+        mod = importlib.util.module_from_spec(spec)
+        sys.modules[name] = mod
+        spec.loader.exec_module(mod)
+    return sys.modules[name]
+
+
+PKG = _package()
+from voxtral_tts_c_amd import session as H  # noqa: E402
+from voxtral_tts_c_amd import synth as S  # noqa: E402
+
+
+class _Checkers:
+    """The CPU checkers: ctypes bindings of oracle/liboracle.so and oracle/_ref/libvoxtral_ref.so and the
+    backends over them, which live with the tests.  Only the cpu_baseline and parity legs below (and the
+    set-up of --workload codec, whose weight-norm reconstruction is the checker's) load them; nothing that
+    is timed on the GPU does."""
+    _mods = None
+
+    def __getattr__(self, name):
+        if _Checkers._mods is None:
+            for d in (os.path.join(ROOT, "tests"), os.path.join(ROOT, "tests", "golden")):
+                if d not in sys.path:
+                    sys.path.insert(0, d)
+                    import codec_cases
+            import codecsupport
+            import vtsupport
+            _Checkers._mods = {"cases": cases, "codec_cases": codec_cases, "codecsupport": codecsupport, "vt": vtsupport}
+        return _Checkers._mods[name]
+
+
+CHK = _Checkers()
+
+
+def BL():
+    """The benchmark companion library (event timing and single-kernel loops on the library's stream)."""
+    return PKG.bench_lib()
 
 HBM_PEAK_GBPS = 8000.0
 N_LAYERS = 26
@@ -109,7 +151,7 @@ def cpu_blas_linears(sgemm, shapes, weights, m, budget_s):
     cblas_sgemm(RowMajor, NoTrans, Trans, seq, out, in, 1, x, in, W, in, 0, y, out).  Times that pair
     for every (out, in) of `shapes` once (twice if the budget allows) on m rows of N(0,1) activations;
     returns the seconds per shape."""
-    orc = S.oracle()
+    orc = CHK.vt.oracle()
     orc.orc_bf16_to_f32_buf.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
     out = {}
     t_start = time.time()
@@ -145,11 +187,10 @@ def cpu_baseline(layers, final_norm, kv_k, kv_v, kv_max, embeds, gpu_hidden, bud
     threads and its decode matvec never reaches BLAS) on the same weights, from
     the same cache state, for as many steps as fit the budget.  Uses the compiled
     reference (oracle/_ref) when it travelled with the tree, else our port."""
-    import cases
     n_cached = PROMPT
-    if S.have_ref():
+    if CHK.vt.have_ref():
         kind = "reference"
-        b = cases.RefBackend()
+        b = CHK.cases.RefBackend()
         b.llm_open(layers, final_norm, kv_max)
         nbytes = N_LAYERS * kv_max * S.KV_DIM * 4
         C.memmove(b.lib.ref_kv_k(b.ctx), kv_k.ctypes.data, nbytes)
@@ -157,7 +198,7 @@ def cpu_baseline(layers, final_norm, kv_k, kv_v, kv_max, embeds, gpu_hidden, bud
         b.lib.ref_set_kv_len(b.ctx, n_cached)
     else:
         kind = "port"
-        b = cases.OracleBackend(threads=1)
+        b = CHK.cases.OracleBackend(threads=1)
         b.llm_open(layers, final_norm, kv_max, n_layers=N_LAYERS)
         b.kv_k[:] = kv_k
         b.kv_v[:] = kv_v
@@ -232,7 +273,6 @@ def prefill_cpu_baseline(layers, budget_s, m=PREFILL_LEN, calls=N_LAYERS):
 def bench_prefill(args):
     """BASELINE.json config "Backbone prefill": 26 layers, 512 random token ids, causal GQA
     attention.  A step is one whole prefill into an empty cache; inputs are resident in HBM."""
-    import cases
     K, W = args.steps, args.warmup
     workers = min(16, os.cpu_count() or 8)
     t0 = time.time()
@@ -251,20 +291,20 @@ def bench_prefill(args):
     for _ in range(W):
         lib.tts_hip_llm_prefill(d_e.ptr, PREFILL_LEN, 0)
     lib.tts_hip_sync()
-    lib.tts_hip_timer_start()
+    BL().tts_hip_timer_start()
     for _ in range(K):
         lib.tts_hip_llm_prefill(d_e.ptr, PREFILL_LEN, 0)
-    ms_step = lib.tts_hip_timer_stop_ms() / K
+    ms_step = BL().tts_hip_timer_stop_ms() / K
     lib.tts_hip_sync()
     hip.check()
     gemm_fl, attn_fl = prefill_flops(PREFILL_LEN)
     # the dominant kernel alone, per projection shape, timed by the library with events
     per_shape = {}
     for i, (name, n, k) in enumerate(GEMM_SHAPES):
-        ms = lib.tts_hip_bench_kernel(i, 50)
+        ms = BL().tts_hip_bench_kernel(i, 50)
         fl = 2.0 * PREFILL_LEN * n * k
         per_shape[name] = {"N": n, "K": k, "us": round(ms * 1e3, 1), "tflops": round(fl / ms / 1e9, 1)}
-    ms_attn = lib.tts_hip_bench_kernel(4, 50)
+    ms_attn = BL().tts_hip_bench_kernel(4, 50)
     hip.check()
     ms_gemm_layer = sum(v["us"] for v in per_shape.values()) / 1e3
     achieved = 2.0 * PREFILL_LEN * LAYER_WEIGHT_ELEMS / ms_gemm_layer / 1e9
@@ -297,10 +337,10 @@ def bench_prefill(args):
     }
     if args.cpu_seconds > 0:
         out["cpu_baseline"] = prefill_cpu_baseline(layers, args.cpu_seconds)
-    if args.cpu_seconds > 0 and S.have_ref():
+    if args.cpu_seconds > 0 and CHK.vt.have_ref():
         # parity of the GPU prefill against the reference's own tts_llm_prefill on the first tokens
         n_cpu = 2
-        b = cases.RefBackend()
+        b = CHK.cases.RefBackend()
         b.llm_open(layers, final_norm, 16)
         t0 = time.time()
         b.llm_prefill(embeds[:n_cpu])
@@ -341,7 +381,6 @@ def acoustic_frame_bytes():
 def bench_acoustic(args):
     """BASELINE.json config "Flow-matching acoustic transformer per frame": 3 layers, batch 2
     (conditional + unconditional, guidance 1.2), 7 Euler steps, FSQ.  A step is one frame."""
-    import cases
     K, W = args.steps, args.warmup
     t0 = time.time()
     ac = S.Acoustic(50)
@@ -351,14 +390,8 @@ def bench_acoustic(args):
     t0 = time.time()
     hip.upload_acoustic(ac)
     t_up = time.time() - t0
-    st = C.c_uint64(0)
-    S.oracle().orc_rng_seed(C.byref(st), 42)
-    hs, xs = [], []
-    for f in range(8):
-        hs.append(S.f32_normal(S.DIM, 20 + f))
-        x0 = np.zeros(S.ACOUSTIC_DIM, np.float32)
-        S.oracle().orc_randn_fill(C.byref(st), S.fp(x0), S.ACOUSTIC_DIM)
-        xs.append(x0)
+    hs = [S.f32_normal(S.DIM, 20 + f) for f in range(8)]
+    xs = [S.f32_normal(S.ACOUSTIC_DIM, 4200 + f) for f in range(8)]      # the frames' noise: any N(0,1) draw
     codes = np.zeros(S.CODES, np.int32)
     d_h = [H.DevBuf.from_numpy(lib, h) for h in hs]
     d_x = [H.DevBuf.from_numpy(lib, x) for x in xs]
@@ -373,10 +406,10 @@ def bench_acoustic(args):
     hip.check()
     per_phase = {}
     for name, which, nbytes in AC_PHASES:
-        ms = lib.tts_hip_bench_kernel(which, 50)
+        ms = BL().tts_hip_bench_kernel(which, 50)
         per_phase[name] = {"us": round(ms * 1e3, 1), "gbps": round(nbytes / ms / 1e6, 1)}
     # the four launches of a layer in order, each turn on the next layer's weights, as inside a frame
-    ms_layer = lib.tts_hip_bench_kernel(14, 60)
+    ms_layer = BL().tts_hip_bench_kernel(14, 60)
     hip.check()
     achieved = AC_LAYER_BYTES / ms_layer / 1e6
     fb = acoustic_frame_bytes()
@@ -417,10 +450,11 @@ def bench_acoustic(args):
     if args.cpu_seconds > 0:
         # parity: as many frames as fit the budget against the CPU port on all host threads (bit-identical
         # to one thread), noise from the restated host RNG at seed 42
-        orc = cases.OracleBackend(threads=min(16, os.cpu_count() or 1))
+        orc = CHK.cases.OracleBackend(threads=min(16, os.cpu_count() or 1))
         orc.ac_open(ac)
         st2 = C.c_uint64(0)
-        S.oracle().orc_rng_seed(C.byref(st2), 42)
+        T = CHK.vt
+        T.oracle().orc_rng_seed(C.byref(st2), 42)
         equal = total = 0
         worst = 0.0
         t0 = time.time()
@@ -430,7 +464,7 @@ def bench_acoustic(args):
             rc, _, rx = orc.acoustic_forward(h, seed=42 if f == 0 else None, want_x=True)
             x0 = np.zeros(S.ACOUSTIC_DIM, np.float32)
             if rc[0] != 1:
-                S.oracle().orc_randn_fill(C.byref(st2), S.fp(x0), S.ACOUSTIC_DIM)
+                T.oracle().orc_randn_fill(C.byref(st2), T.fp(x0), S.ACOUSTIC_DIM)
             g, gx = hip.acoustic_frame(h, x0)
             equal += int(np.sum(g == rc))
             total += S.CODES
@@ -440,16 +474,19 @@ def bench_acoustic(args):
         out["parity"] = {"codes_equal": equal, "codes": total, "frames": f, "max_latent_diff": float(f"{worst:.3e}"),
                          "against": "port", "full_size": "tests/test_gpu_fullsize.py runs all 200 frames (7,400 codes)"}
         assert worst < 1e-4, worst
-    if args.cpu_seconds > 0 and S.have_ref():
+    if args.cpu_seconds > 0 and CHK.vt.have_ref():
         # one frame of the reference's tts_acoustic_forward (14 velocity evaluations), single thread, no BLAS
-        b = cases.RefBackend()
+        b = CHK.cases.RefBackend()
         b.ac_open(ac)
         t0 = time.time()
         rc, _ = b.acoustic_forward(hs[0], seed=42)
         dt = time.time() - t0
         b.ac_close()
-        g = np.zeros(S.CODES, np.int32)
-        lib.tts_hip_acoustic_frame(g.ctypes.data, d_h[0].ptr, d_x[0].ptr, None)
+        st3 = C.c_uint64(0)
+        CHK.vt.oracle().orc_rng_seed(C.byref(st3), 42)
+        x42 = np.zeros(S.ACOUSTIC_DIM, np.float32)
+        CHK.vt.oracle().orc_randn_fill(C.byref(st3), CHK.vt.fp(x42), S.ACOUSTIC_DIM)     # the noise the reference drew
+        g, _ = hip.acoustic_frame(hs[0], x42)
         out["cpu_reference_noblas"] = {"value": round(dt * 1e3, 1), "unit": "ms/frame", "cores": 1, "kind": "reference-noblas",
                                        "sample": "one frame of tts_acoustic_forward at seed 42 (same hidden state and noise)"}
         assert np.array_equal(g, rc), (g, rc)
@@ -480,8 +517,7 @@ def codec_flops(frames):
 def bench_codec(args):
     """Codec decoder: 200 frames of 37 codes (16 s of audio) -> 384,000 samples.  A step is one such
     decode with codes and waveform resident in HBM."""
-    import codecsupport as K
-    import codec_cases as CC
+    K, CC = CHK.codecsupport, CHK.codec_cases      # weight-norm reconstruction of the synthetic weights: the checker's
     Kk, W = args.steps, args.warmup
     t0 = time.time()
     hc = K.HostCodec(5)
@@ -498,17 +534,17 @@ def bench_codec(args):
     for _ in range(W):
         assert lib.tts_hip_codec_decode_device(d_codes.ptr, CODEC_FRAMES, d_wave.ptr) == 0
     lib.tts_hip_sync()
-    lib.tts_hip_timer_start()
+    BL().tts_hip_timer_start()
     for _ in range(Kk):
         lib.tts_hip_codec_decode_device(d_codes.ptr, CODEC_FRAMES, d_wave.ptr)
-    ms_step = lib.tts_hip_timer_stop_ms() / Kk
+    ms_step = BL().tts_hip_timer_stop_ms() / Kk
     hip.check()
     wave = d_wave.to_numpy(np.float32, (CODEC_FRAMES * 1920,))
     shapes = (("qkv 1600x3072x1024", 20, 1600 * 3072 * 1024 * 2), ("wo 1600x1024x1024", 21, 1600 * 1024 * 1024 * 2),
               ("gate|up 1600x8192x1024", 22, 1600 * 8192 * 1024 * 2), ("down 1600x1024x4096", 23, 1600 * 1024 * 4096 * 2))
     per_shape = {}
     for name, which, fl in shapes:
-        ms = lib.tts_hip_bench_kernel(which, 30)
+        ms = BL().tts_hip_bench_kernel(which, 30)
         per_shape[name] = {"us": round(ms * 1e3, 1), "tflops": round(fl / ms / 1e9, 1)}
     hip.check()
     layer_fl = sum(fl for _, _, fl in shapes)
@@ -541,7 +577,7 @@ def bench_codec(args):
         "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
         "cpu_baseline": None,
     }
-    if args.cpu_seconds > 0 and S.have_ref():
+    if args.cpu_seconds > 0 and CHK.vt.have_ref():
         n = 8
         b = CC.RefCodecBackend()
         b.open(hc)
@@ -571,7 +607,6 @@ def bench_frame(args):
     """The whole per-frame loop of voxtral_tts.c:301-321 on the device: 26-layer backbone step,
     acoustic frame (semantic head, 7 guided Euler steps, FSQ) and the audio-code embedding that
     becomes the next backbone input.  A step is one frame; 64-token prompt prefilled first."""
-    import cases
     K, W = args.steps, args.warmup
     workers = min(16, os.cpu_count() or 8)
     t0 = time.time()
@@ -594,11 +629,7 @@ def bench_frame(args):
     assert lib.tts_hip_upload_audio_embeddings(table.ctypes.data, AUDIO_ROWS, offs.ctypes.data) == 0
     t_up = time.time() - t0
     hip.llm_prefill(prompt)
-    st = C.c_uint64(0)
-    S.oracle().orc_rng_seed(C.byref(st), 42)
-    noise = np.zeros((W + K, S.ACOUSTIC_DIM), np.float32)
-    for f in range(W + K):
-        S.oracle().orc_randn_fill(C.byref(st), S.fp(noise[f]), S.ACOUSTIC_DIM)
+    noise = S.f32_normal((W + K, S.ACOUSTIC_DIM), 4200)      # the frames' noise: any N(0,1) draw
     d_e = H.DevBuf.from_numpy(lib, emb_row(24))          # the audio start token's stand-in
     codes = np.zeros(S.CODES, np.int32)
     pos = PROMPT
@@ -646,12 +677,13 @@ def bench_matvec(args):
     """The single bf16 matvec of configs[0]: y = W x, W bf16 ~N(0,0.02), x f32 ~N(0,1), the three
     shapes of the reference's CPU kernel.  A step is one product; launches rotate through copies of
     the two small matrices (8 x 56.6 MB) so that every one streams from HBM, not the memory-side cache."""
-    import cases
     K, W = args.steps, args.warmup
     hip = H.Hip(kv_max=8)
     lib = hip.lib
-    cpu_lib = cases.RefBackend() if S.have_ref() else cases.OracleBackend(threads=1)
-    kind = "reference" if S.have_ref() else "port"
+    cpu_lib = kind = None
+    if args.cpu_seconds > 0:
+        cpu_lib = CHK.cases.RefBackend() if CHK.vt.have_ref() else CHK.cases.OracleBackend(threads=1)
+        kind = "reference" if CHK.vt.have_ref() else "port"
     per_shape, t_gen, t_up = {}, 0.0, 0.0
     cpu_ms, parity = {}, {}
     for n, k, what in MATVEC_SHAPES:
@@ -668,7 +700,7 @@ def bench_matvec(args):
         d_x = H.DevBuf.from_numpy(lib, x)
         d_y = H.DevBuf(lib, 4 * n)
         t_up += time.time() - t0
-        ms = lib.tts_hip_bench_matvec(d_y.ptr, d_x.ptr, d_W.ptr, n * k, copies, k, n, max(K, copies))
+        ms = BL().tts_hip_bench_matvec(d_y.ptr, d_x.ptr, d_W.ptr, n * k, copies, k, n, max(K, copies))
         hip.check()
         got = d_y.to_numpy(np.float32, (1, n))
         name = f"{n}x{k}"
@@ -719,7 +751,6 @@ def bench_layer(args):
     """configs[1]: one decoder layer, decode step at batch 1 over a KV cache of 512 positions
     ~N(0,1).  A step is one tts_hip_layer_decode on a device-resident hidden state (the whole-step
     kernel run over a single layer, final norm off)."""
-    import cases
     K, W = args.steps, args.warmup
     pos, kv_max = 512, 520
     layer = S.Layer(3)
@@ -746,10 +777,10 @@ def bench_layer(args):
     lib.tts_hip_sync()
     # the hidden state is fed back in place: values drift but the bytes moved do not depend on them
     lib.tts_hip_to_device(d_x.ptr, x.ctypes.data, x.nbytes)
-    lib.tts_hip_timer_start()
+    BL().tts_hip_timer_start()
     for _ in range(K):
         lib.tts_hip_layer_decode(0, d_x.ptr, pos)
-    ms = lib.tts_hip_timer_stop_ms() / K
+    ms = BL().tts_hip_timer_stop_ms() / K
     hip.check()
     nbytes = LAYER_WEIGHT_BYTES + 2 * S.DIM * 4 + 2 * (pos + 1) * S.KV_DIM * 4 + 2 * S.KV_DIM * 4 + 2 * S.DIM * 4
     gbps = nbytes / ms / 1e6
@@ -772,9 +803,9 @@ def bench_layer(args):
         "cpu_baseline": None,
     }
     if args.cpu_seconds > 0:
-        kind = "reference" if S.have_ref() else "port"
-        if S.have_ref():
-            b = cases.RefBackend()
+        kind = "reference" if CHK.vt.have_ref() else "port"
+        if CHK.vt.have_ref():
+            b = CHK.cases.RefBackend()
             b.llm_open([layer] * N_LAYERS, ones, kv_max)
             nb = N_LAYERS * kv_max * S.KV_DIM * 4
             C.memmove(b.lib.ref_kv_k(b.ctx), k.ctypes.data, nb)
@@ -786,7 +817,7 @@ def bench_layer(args):
             b.llm_close()
             sample = "one tts_llm_forward over 26 copies of the layer at pos 512, divided by 26"
         else:
-            b = cases.OracleBackend(threads=1)
+            b = CHK.cases.OracleBackend(threads=1)
             b.llm_open([layer], ones, kv_max, n_layers=1)
             b.kv_k[0], b.kv_v[0] = k[0], v[0]
             b.pos = pos
@@ -798,7 +829,7 @@ def bench_layer(args):
                                "sample": sample, "gbps": round(nbytes / cpu_ms / 1e6, 2)}
         # parity of the timed entry point against the CPU port: the port's hidden state is the final
         # norm (unit gains) of the residual stream that tts_hip_layer_decode leaves
-        o = cases.OracleBackend(threads=8)
+        o = CHK.cases.OracleBackend(threads=8)
         o.llm_open([layer], ones, kv_max, n_layers=1)
         o.kv_k[0], o.kv_v[0] = k[0], v[0]
         o.pos = pos
@@ -827,7 +858,7 @@ def other_workloads(hip, kv_max):
         lib.tts_hip_memset(d_W.ptr, 0x3c, copies * 2 * n * k)          # bf16 0x3c3c = 0.0115
         d_x = H.DevBuf.from_numpy(lib, S.f32_normal((1, k), 42))
         d_y = H.DevBuf(lib, 4 * n)
-        ms = lib.tts_hip_bench_matvec(d_y.ptr, d_x.ptr, d_W.ptr, n * k, copies, k, n, 24)
+        ms = BL().tts_hip_bench_matvec(d_y.ptr, d_x.ptr, d_W.ptr, n * k, copies, k, n, 24)
         nbytes = 2 * n * k + 4 * k + 4 * n
         w[f"matvec {n}x{k}"] = {"config": 0, "kernel": "vt_matvec_kernel", "us": round(ms * 1e3, 2), "launches": 24,
                                 "achieved": round(nbytes / ms / 1e6, 1), "unit": "GB/s",
@@ -840,11 +871,11 @@ def other_workloads(hip, kv_max):
     for l in range(N_LAYERS):
         lib.tts_hip_layer_decode(l, d_x.ptr, pos)
     lib.tts_hip_sync()
-    lib.tts_hip_timer_start()
+    BL().tts_hip_timer_start()
     n_l = 2 * N_LAYERS
     for i in range(n_l):
         lib.tts_hip_layer_decode(i % N_LAYERS, d_x.ptr, pos)
-    ms = lib.tts_hip_timer_stop_ms() / n_l
+    ms = BL().tts_hip_timer_stop_ms() / n_l
     nbytes = LAYER_WEIGHT_BYTES + 2 * S.DIM * 4 + 2 * (pos + 1) * S.KV_DIM * 4 + 2 * S.KV_DIM * 4 + 2 * S.DIM * 4
     w["layer decode, 512 cached positions"] = {
         "config": 1, "kernel": "vt_decode_step_kernel (one layer per launch)", "us": round(ms * 1e3, 2), "launches": n_l,
@@ -855,26 +886,23 @@ def other_workloads(hip, kv_max):
     for _ in range(3):
         lib.tts_hip_llm_prefill(d_e.ptr, PREFILL_LEN, 0)
     lib.tts_hip_sync()
-    lib.tts_hip_timer_start()
+    BL().tts_hip_timer_start()
     for _ in range(8):
         lib.tts_hip_llm_prefill(d_e.ptr, PREFILL_LEN, 0)
-    ms = lib.tts_hip_timer_stop_ms() / 8
+    ms = BL().tts_hip_timer_stop_ms() / 8
     gemm_fl, attn_fl = prefill_flops(PREFILL_LEN)
-    ms_layer = sum(lib.tts_hip_bench_kernel(i, 26) for i in range(4))
+    ms_layer = sum(BL().tts_hip_bench_kernel(i, 26) for i in range(4))
     achieved = 2.0 * PREFILL_LEN * LAYER_WEIGHT_ELEMS / ms_layer / 1e9
     w["prefill, 512 tokens x 26 layers"] = {
         "config": 3, "kernel": "vt_gemm_wide_kernel (the projection launches of one layer)", "ms": round(ms, 3), "launches": 8,
         "tokens_per_s": round(PREFILL_LEN / (ms * 1e-3), 1), "tflops_whole_prefill": round((gemm_fl + attn_fl) / ms / 1e9, 1),
         "us_products_per_layer": round(ms_layer * 1e3, 1), "achieved": round(achieved, 1), "unit": "TFLOP/s",
-        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "attention_us_per_layer": round(lib.tts_hip_bench_kernel(4, 26) * 1e3, 1)}
+        "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4), "attention_us_per_layer": round(BL().tts_hip_bench_kernel(4, 26) * 1e3, 1)}
     d_e.free()
     # configs[4]
     ac = S.Acoustic(50)
     hip.upload_acoustic(ac)
-    st = C.c_uint64(0)
-    S.oracle().orc_rng_seed(C.byref(st), 42)
-    x0 = np.zeros(S.ACOUSTIC_DIM, np.float32)
-    S.oracle().orc_randn_fill(C.byref(st), S.fp(x0), S.ACOUSTIC_DIM)
+    x0 = S.f32_normal(S.ACOUSTIC_DIM, 4200)
     d_h, d_x0 = H.DevBuf.from_numpy(lib, S.f32_normal(S.DIM, 20)), H.DevBuf.from_numpy(lib, x0)
     codes = np.zeros(S.CODES, np.int32)
     for _ in range(2):
@@ -883,12 +911,82 @@ def other_workloads(hip, kv_max):
     for _ in range(10):
         lib.tts_hip_acoustic_frame(codes.ctypes.data, d_h.ptr, d_x0.ptr, None)
     ms = (time.perf_counter() - t0) * 1e3 / 10
-    ms_layer = lib.tts_hip_bench_kernel(14, 30)
+    ms_layer = BL().tts_hip_bench_kernel(14, 30)
     achieved = AC_LAYER_BYTES / ms_layer / 1e6
     w["acoustic frame"] = {
         "config": 4, "kernel": "vt_ac_phase_kernel (the launches of one layer, in order)", "ms": round(ms, 4), "launches": 10,
         "frame_gbps": round(acoustic_frame_bytes() / ms / 1e6, 1), "us_per_layer": round(ms_layer * 1e3, 1),
         "achieved": round(achieved, 1), "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4)}
+    # configs[2] at the cache lengths of a real utterance (~250 prompt rows + up to 2000 frames): the whole-step
+    # kernel at a fixed position over K and V rows filled by a kernel with pseudo-random values
+    ctx = PKG.ctx()
+    d_e, d_hid = H.DevBuf.from_numpy(lib, S.f32_normal(S.DIM, 43)), H.DevBuf(lib, S.DIM * 4)
+    for pos in (1024, 2000):
+        if pos + 1 > kv_max:
+            continue
+        for base in (ctx.kv_cache_k_gpu, ctx.kv_cache_v_gpu):
+            for l in range(N_LAYERS):
+                BL().tts_hip_bench_fill_f32(base + l * kv_max * S.KV_DIM * 4, pos * S.KV_DIM)
+        for _ in range(3):
+            lib.tts_hip_llm_forward_device(d_hid.ptr, d_e.ptr, pos)
+        lib.tts_hip_sync()
+        BL().tts_hip_timer_start()
+        n_l = 12
+        for _ in range(n_l):
+            lib.tts_hip_llm_forward_device(d_hid.ptr, d_e.ptr, pos)
+        ms = BL().tts_hip_timer_stop_ms() / n_l
+        nb = step_bytes(pos)
+        assert np.all(np.isfinite(d_hid.to_numpy(np.float32, S.DIM)))
+        w[f"decode @{pos} cached positions"] = {
+            "config": 2, "kernel": "vt_decode_step_kernel", "ms": round(ms, 4), "launches": n_l, "bytes_per_launch": int(nb),
+            "achieved": round(nb / ms / 1e6, 1), "unit": "GB/s", "frac": round(nb / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+    # the generation loop (voxtral_tts.c:301-321) on the device: backbone step + acoustic frame + code embedding
+    table = S.bf16_normal((AUDIO_ROWS, S.DIM), 4242, 0.05)
+    offs = np.zeros(S.CODES, np.int32)
+    offs[1] = 8194
+    for i in range(2, S.CODES):
+        offs[i] = offs[i - 1] + 23
+    assert lib.tts_hip_upload_audio_embeddings(table.ctypes.data, AUDIO_ROWS, offs.ctypes.data) == 0
+    noise = S.f32_normal((16, S.ACOUSTIC_DIM), 4300)
+    lib.tts_hip_to_device(d_e.ptr, emb_row(24).ctypes.data, S.DIM * 4)
+    pos, n_f = PROMPT, 12
+    for f in range(4):
+        lib.tts_hip_generate_frame(codes.ctypes.data, d_e.ptr, noise[f].ctypes.data, pos + f)
+    t0 = time.perf_counter()
+    for f in range(4, 4 + n_f):
+        lib.tts_hip_generate_frame(codes.ctypes.data, d_e.ptr, noise[f].ctypes.data, pos + f)
+    ms = (time.perf_counter() - t0) * 1e3 / n_f
+    fb = step_bytes(pos + 4 + (n_f - 1) / 2.0) + acoustic_frame_bytes() + S.CODES * S.DIM * 2
+    w["generation loop (backbone step + acoustic frame + code embedding)"] = {
+        "config": "2+4", "kernel": "vt_decode_step_kernel + vt_ac_phase_kernel launches", "ms": round(ms, 4), "launches": n_f,
+        "frames_per_s": round(1000.0 / ms, 1), "realtime_factor": round(FRAME_SECONDS * 1000.0 / ms, 1),
+        "bytes_per_frame": int(fb), "achieved": round(fb / ms / 1e6, 1), "unit": "GB/s",
+        "frac": round(fb / ms / 1e6 / HBM_PEAK_GBPS, 4), "timed": "host clock, one synchronisation per frame"}
+    for b in (d_e, d_hid):
+        b.free()
+    # the codec decoder on 200 frames (16 s of audio), codes and waveform resident
+    cw = S.CodecWeights(5)
+    cs = cw.struct()
+    assert lib.tts_hip_upload_codec_weights(C.addressof(cs)) == 0, lib.tts_hip_last_error()
+    d_codes = H.DevBuf.from_numpy(lib, cw.random_codes(CODEC_FRAMES, 77))
+    d_wave = H.DevBuf(lib, CODEC_FRAMES * 1920 * 4)
+    for _ in range(2):
+        assert lib.tts_hip_codec_decode_device(d_codes.ptr, CODEC_FRAMES, d_wave.ptr) == 0
+    lib.tts_hip_sync()
+    BL().tts_hip_timer_start()
+    for _ in range(6):
+        lib.tts_hip_codec_decode_device(d_codes.ptr, CODEC_FRAMES, d_wave.ptr)
+    ms = BL().tts_hip_timer_stop_ms() / 6
+    assert np.all(np.isfinite(d_wave.to_numpy(np.float32, (CODEC_FRAMES * 1920,))))
+    ms_l = sum(BL().tts_hip_bench_kernel(k, 12) for k in (20, 21, 22, 23))
+    fl_l = 2.0 * 1600 * 1024 * (3072 + 1024 + 8192 + 4096)
+    w["codec decode, 200 frames"] = {
+        "config": "N4", "kernel": "vt_codec_gemm_kernel (the four products of a last-stage layer)", "ms": round(ms, 4), "launches": 6,
+        "tflops_whole_decode": round(codec_flops(CODEC_FRAMES) / ms / 1e9, 1),
+        "times_real_time": round(CODEC_FRAMES * FRAME_SECONDS * 1e3 / ms, 1), "us_products_per_layer": round(ms_l * 1e3, 1),
+        "achieved": round(fl_l / ms_l / 1e9, 1), "unit": "TFLOP/s", "frac": round(fl_l / ms_l / 1e9 / MFMA_F32_PEAK_TFLOPS, 4)}
+    for b in (d_codes, d_wave):
+        b.free()
     hip.check()
     return w
 
@@ -939,6 +1037,8 @@ def main():
 
     n_cpu = 6 if args.cpu_seconds > 0 else 0
     kv_max = max(PROMPT + n_cpu + 2 * (W + K) + 8, PREFILL_LEN + 8)     # room for the 512-row workloads below
+    if not args.no_workloads:
+        kv_max = max(kv_max, 2008)                                      # and for the decode workload at 2000 positions
     hip = H.Hip(kv_max=kv_max)
     lib = hip.lib
     lib.tts_hip_set_decode_mode(args.mode)
@@ -990,9 +1090,9 @@ def main():
     run(W, True)
     lib.tts_hip_sync()
     pos0 = pos
-    lib.tts_hip_timer_start()
+    BL().tts_hip_timer_start()
     run(K, True)
-    ms_total = lib.tts_hip_timer_stop_ms()
+    ms_total = BL().tts_hip_timer_stop_ms()
     lib.tts_hip_sync()
     hip.check()
     ms_step = ms_total / K
@@ -1004,10 +1104,16 @@ def main():
     run(min(W, 5), False)
     pos = pos0
     lib.tts_hip_sync()
-    lib.tts_hip_timer_start()
+    BL().tts_hip_timer_start()
     run(K, False)
-    ms_kernel = lib.tts_hip_timer_stop_ms() / K
+    ms_kernel = BL().tts_hip_timer_stop_ms() / K
     lib.tts_hip_sync()
+    hip.check()
+
+    # what a grid of this shape can stream at all: the same grid, per-wave shares, loads and ring depth over the
+    # same 26 layers of weights, with no arithmetic, staging or hand-overs
+    nbytes_c = C.c_double(0.0)
+    ms_ceiling = BL().tts_hip_bench_stream_ceiling(max(3, min(K, 20)), C.byref(nbytes_c))
     hip.check()
 
     # the drop-in entry point with host pointers (12 KB up, 12 KB down and one synchronisation per
@@ -1059,6 +1165,11 @@ def main():
             "traffic_source": TRAFFIC_SOURCE if args.traffic_kib is None else "--traffic-kib",
             "bytes_per_launch": int(bytes_launch),
             "ms_per_launch": round(ms_kernel, 4),
+            "stream_ceiling_gbps": round(nbytes_c.value / ms_ceiling / 1e6, 1),
+            "stream_ceiling_ms": round(ms_ceiling, 4),
+            "frac_of_stream_ceiling": round(achieved / (nbytes_c.value / ms_ceiling / 1e6), 4),
+            "stream_ceiling": "a plain streaming kernel with this kernel's grid, per-wave shares, 16-byte non-temporal "
+                              "loads and 18 loads in flight per wave over the same 26 layers of weights",
         },
         "setup_s": {"generate": round(t_gen, 1), "upload": round(t_up, 1)},
     }

@@ -290,7 +290,7 @@ void tts_hip_set_decode_mode(int mode);
  * invalid.  Entry points with host pointers (tts_hip_llm_forward, tts_hip_generate_frame) report
  * that themselves; after the asynchronous ones (tts_hip_llm_forward_device, tts_hip_layer_decode)
  * it is reported, once, by the next call that waits for the stream: tts_hip_sync, tts_hip_to_host,
- * tts_hip_to_device, tts_hip_memset, tts_hip_timer_stop_ms (which then returns a negative time).
+ * tts_hip_to_device, tts_hip_memset.
  * The report resets the barrier; the next step starts clean. */
 void tts_hip_set_barrier_timeout(unsigned long long ticks);
 /* Workgroups of the backbone's whole-step decode kernel: 0 (the default) = the CU count rounded down to
@@ -307,27 +307,6 @@ void tts_hip_set_acoustic_grid(int workgroups);
 int tts_hip_error_count(void);
 const char *tts_hip_last_error(void);
 
-/* Event timing on the internal stream (for benchmarks). */
-void tts_hip_timer_start(void);
-float tts_hip_timer_stop_ms(void);
-/* Average duration in ms of one launch of a single kernel, timed with events on the
- * internal stream over `iters` launches on pseudo-random activations of normal size (on zeros
- * the matrix cores draw less power and the products measure 5-15 % faster than in a real pass;
- * needs the weights uploaded; launch i takes the weights of uploaded layer i modulo their
- * number, so that they come from HBM as in a real pass): which 0..3 = sequence-level product at M = 512 with the
- * q|k|v, output, gate/up and down projection; 4 = causal attention at 512 queries (KV cache
- * of at least 512 rows); 10..13 = the four acoustic phase kernels, 14 = the four of them in
- * order on one layer (the value is the duration of all four); 20..23 = the codec's fp32
- * product at 1600 rows with the q|k|v, output, gate|up and down matrices, 24 = the whole codec
- * decoder on 200 frames (codec weights uploaded).  Negative on error. */
-float tts_hip_bench_kernel(int which, int iters);
-/* Average duration in ms of one single-row product y[out_dim] = W[out_dim, in_dim] x (the kernel
- * behind tts_hip_linear_bf16 with seq_len 1), timed with events on the internal stream over
- * `iters` launches.  Launch i reads copy i % n_copies of W, `copy_stride` elements apart, so that
- * a matrix smaller than the memory-side cache is streamed from HBM every time.  Device pointers.
- * Negative on error. */
-float tts_hip_bench_matvec(float *d_y, const float *d_x, const uint16_t *d_W, size_t copy_stride,
-                           int n_copies, int in_dim, int out_dim, int iters);
 /* The activation format of the sequence-level products: n fp32 values (n even, device pointers,
  * 8-byte aligned) -> two bf16 planes, hi = bf16(x) rounded to nearest even and lo = bf16(x - hi),
  * so that hi + lo carries x to about 2^-17 relative (tts_hip_linear_bf16 with seq_len >= 8 and

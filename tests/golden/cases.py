@@ -48,10 +48,10 @@ class RefBackend:
         self.lib.tts_apply_rope(S.fp(x), S.fp(freqs), seq, heads, S.HEAD_DIM)
         return x
 
-    def causal_attention(self, Q, K, V, seq_q, seq_k, q_offset):
+    def causal_attention(self, Q, K, V, seq_q, seq_k, q_offset, heads=S.HEADS, kv_heads=S.KV_HEADS):
         out = np.zeros_like(Q)
         self.lib.tts_causal_attention(S.fp(out), S.fp(Q), S.fp(K), S.fp(V), seq_q, seq_k,
-                                      S.HEADS, S.KV_HEADS, S.HEAD_DIM,
+                                      heads, kv_heads, S.HEAD_DIM,
                                       1.0 / np.sqrt(np.float32(S.HEAD_DIM)), 0, q_offset)
         return out
 
@@ -178,10 +178,10 @@ class OracleBackend:
         self.lib.orc_apply_rope(S.fp(x), S.fp(freqs), seq, heads, S.HEAD_DIM)
         return x
 
-    def causal_attention(self, Q, K, V, seq_q, seq_k, q_offset):
+    def causal_attention(self, Q, K, V, seq_q, seq_k, q_offset, heads=S.HEADS, kv_heads=S.KV_HEADS):
         out = np.zeros_like(Q)
         self.lib.orc_causal_attention(S.fp(out), S.fp(Q), S.fp(K), S.fp(V), seq_q, seq_k,
-                                      S.HEADS, S.KV_HEADS, S.HEAD_DIM,
+                                      heads, kv_heads, S.HEAD_DIM,
                                       1.0 / np.sqrt(np.float32(S.HEAD_DIM)), 0, q_offset)
         return out
 

@@ -15,8 +15,8 @@ pytestmark = pytest.mark.skipif(not os.path.exists(pkg.LIB_PATH),
                                 reason="library not built (run __graft_entry__.build())")
 
 
-def declared_symbols():
-    text = open(os.path.join(S.ROOT, "include", "voxtral_tts_hip.h")).read()
+def declared_symbols(header="voxtral_tts_hip.h"):
+    text = open(os.path.join(S.ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(tts_hip_[a-z0-9_]+)\s*\(", text)))
 
@@ -30,6 +30,20 @@ def test_every_declared_symbol_is_exported_and_typed():
         assert n in pkg.SIGNATURES, f"{n} has no ctypes signature"
     assert set(pkg.SIGNATURES) == set(names)
     assert pkg.ctx().initialized in (0, 1)
+
+
+def test_bench_companion_exports_its_header_and_nothing_of_it_is_in_the_product():
+    """Timing loops live in libvoxtral_tts_hip_bench.so (include/voxtral_tts_hip_bench.h); the product
+    library's header declares none of them."""
+    names = declared_symbols("voxtral_tts_hip_bench.h")
+    assert set(names) == set(pkg.BENCH_SIGNATURES)
+    bl = pkg.bench_lib()
+    product = C.CDLL(pkg.LIB_PATH)
+    for n in names:
+        assert hasattr(bl, n), n
+        assert n not in pkg.SIGNATURES
+        assert not hasattr(product, n), f"{n} is still exported by the product library"
+    assert not (set(declared_symbols()) & set(names))
 
 
 def test_host_structs_match_the_reference_layout():

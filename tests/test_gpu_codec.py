@@ -76,6 +76,25 @@ def test_waveform_matches_the_oracle(session, n_frames):
     print(f"n_frames {n_frames}: max|d|/rms {worst:.2e}, rel l2 {l2:.2e}")
 
 
+@pytest.mark.timeout(900)
+def test_waveform_of_a_200_frame_utterance_matches_the_oracle(session):
+    """The size the benchmark times (16 s of audio; tts_codec_decode, voxtral_tts_codec.c:389-503): the
+    200- and 400-row stages under-fill the product kernel's 128-row tiles and K is cut differently than
+    at a few frames, so the whole utterance is compared, and every second of it on its own."""
+    hip, cs = session
+    n_frames = 200
+    codes = K.random_codes(n_frames, 300)
+    print("codec oracle on 200 frames ...", flush=True)
+    ref = K.oracle_decode(cs, codes)
+    got = hip_decode(hip, codes)
+    assert got.size == n_frames * 1920
+    worst, l2 = check(ref, got)
+    per_s = 24000
+    for i in range(0, ref.size, per_s):
+        check(ref[i:i + per_s], got[i:i + per_s])
+    print(f"n_frames {n_frames}: max|d|/rms {worst:.2e}, rel l2 {l2:.2e}")
+
+
 def test_repeat_and_shrink_are_reproducible(session):
     hip, cs = session
     codes = K.random_codes(24, 7)

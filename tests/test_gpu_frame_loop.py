@@ -153,5 +153,10 @@ def test_abandoned_backbone_step_fails_the_frame(session):
     hip.check()
     orc.pos = 0
     h = orc.llm_forward(e)
-    ref_codes, _ = hip.acoustic_frame(h, x0)          # the frame kernels on the oracle's hidden state
-    assert codes[0] == ref_codes[0] and int(np.sum(codes != ref_codes)) <= 1, (codes, ref_codes)
+    ref_codes, ref_x = hip.acoustic_frame(h, x0)      # the frame kernels on the oracle's hidden state
+    assert codes[0] == ref_codes[0], (codes, ref_codes)
+    # the two hidden states differ by the backbone's summation noise: a code may differ by one level, and
+    # only where the latent lies on a rounding boundary (the rule of test_generation_loop above)
+    for i in np.nonzero(codes[1:] != ref_codes[1:])[0]:
+        assert abs(int(codes[1 + i]) - int(ref_codes[1 + i])) == 1, (i, codes[1 + i], ref_codes[1 + i])
+        assert fsq_margin(ref_x[i]) < FSQ_NOISE, (i, fsq_margin(ref_x[i]))

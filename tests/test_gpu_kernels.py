@@ -182,10 +182,29 @@ def test_causal_attention_prefill_with_offset(hip, orc):
                                              S.KV_HEADS, S.HEAD_DIM, SCALE)
     hip.lib.tts_hip_sync()
     ref = orc.causal_attention(Q, K, V, seq, start + seq, start)
-    # the sequence kernel feeds (hi, lo) bf16 pairs to the matrix cores (16 mantissa bits per operand):
-    # the reference's rule with the absolute floor scaled to the output, as for the seq > 1 linear
+    # 8 or more queries with the model's head counts run on the matrix cores, which are fed (hi, lo) bf16
+    # pairs (16 mantissa bits per operand): the reference's rule with the absolute floor scaled to the
+    # output, as for the seq > 1 linear
     ok, mr, ma, bad = S.compare_tensors(ref, dO.to_numpy(np.float32, Q.shape), 1e-3,
                                         1e-3 * float(np.sqrt(np.mean(ref.astype(np.float64) ** 2))))
+    assert ok, (mr, ma, bad)
+
+
+@pytest.mark.parametrize("seq,start,heads,kv_heads", [(5, 3, S.HEADS, S.KV_HEADS), (12, 5, 8, 2), (7, 0, 4, 4)])
+def test_causal_attention_prefill_fp32_path(hip, orc, seq, start, heads, kv_heads):
+    """Fewer than 8 queries, or head counts other than the model's, take the fp32 row kernel: the
+    reference's own tolerances for its decode attention apply unchanged (test_kernels.c:168-232,
+    rtol 1e-3 / atol 1e-5)."""
+    Q = S.f32_normal((seq, heads * S.HEAD_DIM), 410 + seq)
+    K = S.f32_normal((start + seq, kv_heads * S.HEAD_DIM), 411 + seq)
+    V = S.f32_normal((start + seq, kv_heads * S.HEAD_DIM), 412 + seq)
+    dQ, dK, dV, dO = dev(hip, Q), dev(hip, K), dev(hip, V), H.DevBuf(hip.lib, Q.nbytes)
+    hip.lib.tts_hip_causal_attention_prefill(dO.ptr, dQ.ptr, dK.ptr, dV.ptr, seq, start, heads,
+                                             kv_heads, S.HEAD_DIM, SCALE)
+    hip.lib.tts_hip_sync()
+    hip.check()
+    ref = orc.causal_attention(Q, K, V, seq, start + seq, start, heads=heads, kv_heads=kv_heads)
+    ok, mr, ma, bad = S.compare_tensors(ref, dO.to_numpy(np.float32, Q.shape), 1e-3, 1e-5)
     assert ok, (mr, ma, bad)
 
 

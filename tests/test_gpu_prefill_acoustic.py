@@ -185,14 +185,14 @@ def test_single_kernel_timing_modes(ac_session):
     in-order figure lies between the largest phase and a generous multiple of their
     sum, and an unknown selector is an error, not a launch."""
     hip, orc, ac = ac_session
-    alone = [hip.lib.tts_hip_bench_kernel(w, 5) for w in (10, 11, 12, 13)]
-    layer = hip.lib.tts_hip_bench_kernel(14, 5)
+    alone = [hip.pkg.bench_lib().tts_hip_bench_kernel(w, 5) for w in (10, 11, 12, 13)]
+    layer = hip.pkg.bench_lib().tts_hip_bench_kernel(14, 5)
     hip.check()
     assert all(0.0 < a < 1.0 for a in alone), alone
     assert max(alone) < layer < 3.0 * sum(alone), (alone, layer)
     n0 = hip.lib.tts_hip_error_count()
-    assert hip.lib.tts_hip_bench_kernel(15, 5) < 0
-    assert hip.lib.tts_hip_bench_kernel(14, 0) < 0
+    assert hip.pkg.bench_lib().tts_hip_bench_kernel(15, 5) < 0
+    assert hip.pkg.bench_lib().tts_hip_bench_kernel(14, 0) < 0
     assert hip.lib.tts_hip_error_count() == n0 + 2
     hip.err0 = n0 + 2                                      # the two errors above were asked for
     # the frame still runs after the timing loops used the same work buffers

@@ -6,8 +6,10 @@ The oracle is test infrastructure: it is only ever loaded from here (tests),
 from the smoke check and from the benchmark's cpu_baseline leg.
 """
 import ctypes as C
+import importlib.util
 import os
 import subprocess
+import sys
 
 import numpy as np
 
@@ -15,10 +17,27 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 GOLDEN_DIR = os.path.join(ROOT, "tests", "golden")
 
-DIM, HEADS, KV_HEADS, HEAD_DIM = 3072, 32, 8, 128
-Q_DIM, KV_DIM, FFN = 4096, 1024, 9216
-EPS, THETA = 1e-5, 1000000.0
-ACOUSTIC_DIM, SEM_PADDED, CODES = 36, 8320, 37
+PKG_DIR = os.path.join(ROOT, "voxtral-tts.c_amd")
+
+
+def load_package():
+    """Import the package directory (its name is not a Python identifier)."""
+    name = "voxtral_tts_c_amd"
+    if name in sys.modules:
+        return sys.modules[name]
+    spec = importlib.util.spec_from_file_location(
+        name, os.path.join(PKG_DIR, "__init__.py"), submodule_search_locations=[PKG_DIR])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+load_package()
+from voxtral_tts_c_amd import synth as _synth  # noqa: E402
+from voxtral_tts_c_amd.synth import (  # noqa: E402,F401  (the seeded generators and metrics, shared with bench.py)
+    DIM, HEADS, KV_HEADS, HEAD_DIM, Q_DIM, KV_DIM, FFN, EPS, THETA, ACOUSTIC_DIM, SEM_PADDED, CODES,
+    f32_to_bf16_trunc, bf16_to_f32, bf16_normal, f32_normal, norm_weight, Layer, rel_errors, compare_tensors)
 
 f32p = C.POINTER(C.c_float)
 u16p = C.POINTER(C.c_uint16)
@@ -39,70 +58,6 @@ def up(a):
 def ip(a):
     assert a.dtype == np.int32 and a.flags["C_CONTIGUOUS"]
     return a.ctypes.data_as(i32p)
-
-
-# --------------------------------------------------------------------------
-# synthetic data
-# --------------------------------------------------------------------------
-
-def f32_to_bf16_trunc(a):
-    """bf16 by truncation (bits >> 16), as the reference test does
-    (test_kernels.c:68-76)."""
-    a = np.ascontiguousarray(a, dtype=np.float32)
-    return (a.view(np.uint32) >> 16).astype(np.uint16)
-
-
-def bf16_to_f32(h):
-    return (h.astype(np.uint32) << 16).view(np.float32)
-
-
-def bf16_normal(shape, seed, std=0.02):
-    g = np.random.default_rng(seed)
-    return f32_to_bf16_trunc(g.standard_normal(shape, dtype=np.float32) * np.float32(std))
-
-
-def f32_normal(shape, seed, std=1.0):
-    g = np.random.default_rng(seed)
-    return (g.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
-
-
-def norm_weight(n, seed):
-    """Positive RMSNorm gains |N(0,1)|*0.1+0.01 in the style of the reference
-    test's fill_random_positive (test_kernels.c:62-66); O(1) after scaling so
-    that hidden states stay O(1) through many layers."""
-    g = np.random.default_rng(seed)
-    return (np.abs(g.standard_normal(n, dtype=np.float32)) * np.float32(0.5)
-            + np.float32(0.75)).astype(np.float32)
-
-
-class Layer:
-    """One transformer layer of synthetic weights (numpy, host)."""
-    FIELDS = ("wq", "wk", "wv", "wo", "w1", "w2", "w3")
-    SHAPES = dict(wq=(Q_DIM, DIM), wk=(KV_DIM, DIM), wv=(KV_DIM, DIM), wo=(DIM, Q_DIM),
-                  w1=(FFN, DIM), w2=(DIM, FFN), w3=(FFN, DIM))
-
-    def __init__(self, seed, std=0.02):
-        for i, f in enumerate(self.FIELDS):
-            setattr(self, f, bf16_normal(self.SHAPES[f], seed * 16 + i, std))
-        self.attention_norm = norm_weight(DIM, seed * 16 + 8)
-        self.ffn_norm = norm_weight(DIM, seed * 16 + 9)
-
-
-class Acoustic:
-    """Synthetic acoustic-transformer weights (numpy, host)."""
-
-    def __init__(self, seed, n_layers=3, bias=True, std=0.02):
-        self.n_layers = n_layers
-        self.layers = [Layer(seed + 1 + i, std) for i in range(n_layers)]
-        self.time_inv_freq = np.zeros(DIM // 2, np.float32)
-        oracle().orc_default_time_inv_freq(fp(self.time_inv_freq), DIM // 2)
-        self.input_proj = bf16_normal((DIM, ACOUSTIC_DIM), seed * 16 + 1, 0.2)
-        self.time_proj = bf16_normal((DIM, DIM), seed * 16 + 2, std)
-        self.llm_proj = bf16_normal((DIM, DIM), seed * 16 + 3, std)
-        self.semantic_out = bf16_normal((SEM_PADDED, DIM), seed * 16 + 4, std)
-        self.semantic_out_bias = f32_normal(SEM_PADDED, seed * 16 + 5, 0.1) if bias else None
-        self.acoustic_out = bf16_normal((ACOUSTIC_DIM, DIM), seed * 16 + 6, std)
-        self.norm = norm_weight(DIM, seed * 16 + 7)
 
 
 # --------------------------------------------------------------------------
@@ -277,28 +232,13 @@ def ref_bind_acoustic(ctx, ac):
                        fp(ac.norm))
 
 
-# --------------------------------------------------------------------------
-# comparison metrics
-# --------------------------------------------------------------------------
+class Acoustic(_synth.Acoustic):
+    """Synthetic acoustic-transformer weights whose time-embedding table is the oracle's
+    (orc_default_time_inv_freq), so that oracle, compiled reference and GPU get the same one."""
 
-def rel_errors(ref_v, test_v):
-    """(max|d|/rms(ref), ||d||2/||ref||2) for one hidden-state vector."""
-    ref_v = np.asarray(ref_v, np.float64).ravel()
-    test_v = np.asarray(test_v, np.float64).ravel()
-    d = test_v - ref_v
-    rms = np.sqrt(np.mean(ref_v ** 2)) + 1e-30
-    return float(np.max(np.abs(d)) / rms), float(np.linalg.norm(d) / (np.linalg.norm(ref_v) + 1e-30))
+    def __init__(self, seed, n_layers=3, bias=True, std=0.02):
+        t = np.zeros(DIM // 2, np.float32)
+        oracle().orc_default_time_inv_freq(fp(t), DIM // 2)
+        super().__init__(seed, n_layers, bias, std, time_inv_freq=t)
 
 
-def compare_tensors(ref_v, test_v, rtol, atol):
-    """The reference's rtol-OR-atol rule (test_kernels.c:79-116): an element
-    is bad iff rel > rtol and |d| > atol; pass iff no bad element and
-    (max_rel <= rtol or max_abs <= atol)."""
-    ref_v = np.asarray(ref_v, np.float32).ravel()
-    test_v = np.asarray(test_v, np.float32).ravel()
-    diff = np.abs(ref_v - test_v)
-    denom = np.maximum(np.abs(ref_v), np.float32(1e-8))
-    rel = diff / denom
-    n_bad = int(np.sum((rel > rtol) & (diff > atol)))
-    ok = (rel.max() <= rtol or diff.max() <= atol) and n_bad == 0
-    return bool(ok), float(rel.max()), float(diff.max()), n_bad

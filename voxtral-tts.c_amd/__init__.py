@@ -113,10 +113,6 @@ SIGNATURES = {
     "tts_hip_set_decode_mode": (None, [C.c_int]),
     "tts_hip_error_count": (C.c_int, []),
     "tts_hip_last_error": (C.c_char_p, []),
-    "tts_hip_timer_start": (None, []),
-    "tts_hip_timer_stop_ms": (C.c_float, []),
-    "tts_hip_bench_kernel": (C.c_float, [C.c_int, C.c_int]),
-    "tts_hip_bench_matvec": (C.c_float, [vp, vp, vp, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int]),
     "tts_hip_split_planes": (C.c_int, [vp, vp, vp, C.c_size_t]),
     "tts_hip_upload_audio_embeddings": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p]),
     "tts_hip_audio_embed": (None, [C.c_void_p, C.c_void_p]),
@@ -134,7 +130,20 @@ SIGNATURES = {
                                             C.c_void_p, C.c_void_p]),
 }
 
+# every symbol include/voxtral_tts_hip_bench.h declares (csrc/libvoxtral_tts_hip_bench.so, the benchmark
+# companion: timing loops around the product's own launches; links against the library above)
+BENCH_LIB_PATH = os.path.join(os.path.dirname(LIB_PATH), "libvoxtral_tts_hip_bench.so")
+BENCH_SIGNATURES = {
+    "tts_hip_timer_start": (None, []),
+    "tts_hip_timer_stop_ms": (C.c_float, []),
+    "tts_hip_bench_kernel": (C.c_float, [C.c_int, C.c_int]),
+    "tts_hip_bench_matvec": (C.c_float, [vp, vp, vp, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "tts_hip_bench_stream_ceiling": (C.c_float, [C.c_int, C.POINTER(C.c_double)]),
+    "tts_hip_bench_fill_f32": (C.c_int, [vp, C.c_size_t]),
+}
+
 _lib = None
+_bench_lib = None
 
 
 def build(force=False):
@@ -160,6 +169,22 @@ def lib():
             fn.argtypes = args
         _lib = l
     return _lib
+
+
+def bench_lib():
+    """The benchmark companion library (shares the product library's context)."""
+    global _bench_lib
+    if _bench_lib is None:
+        lib()                              # the product library first: the companion links against it
+        if not os.path.exists(BENCH_LIB_PATH):
+            raise RuntimeError(f"{BENCH_LIB_PATH} is not built; run `make -C {CSRC}`")
+        l = C.CDLL(BENCH_LIB_PATH)
+        for name, (res, args) in BENCH_SIGNATURES.items():
+            fn = getattr(l, name)
+            fn.restype = res
+            fn.argtypes = args
+        _bench_lib = l
+    return _bench_lib
 
 
 def ctx():

@@ -677,33 +677,26 @@ static int run_layers(const ac_work *w) {
     return 0;
 }
 
-/* average duration (ms) of one launch of phase `phase` of acoustic layer 0 on the work area */
-float vt_bench_acoustic_phase(int phase, int iters) {
-    if (!g_vt.initialized || !g_vt.ac_uploaded) { vt_set_error("bench: acoustic weights not uploaded"); return -1.f; }
+/* For other translation units of the library: the four phase launches of acoustic layer `layer` on
+ * the work area (phase 0..3 = that launch alone, 4 = all four in order), and the work area itself. */
+int vt_ac_launch_layer_phase(int layer, int phase) {
+    if (!g_vt.initialized || !g_vt.ac_uploaded) { vt_set_error("acoustic weights not uploaded"); return -1; }
     float *base = (float *)vt_scratch(sizeof(float) * AC_WORK_FLOATS);
-    if (!base) return -1.f;
+    if (!base || layer < 0 || layer >= TTS_HIP_AC_LAYERS) return -1;
     ac_work w;
     carve(&w, base);
-    if (vt_check(hipMemsetAsync(base, 0, sizeof(float) * AC_WORK_FLOATS, g_vt.stream), "bench clear")) return -1.f;
-    float ms = -1.f;
-    for (int it = -2; it < iters; it++) {
-        if (it == 0 && vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench start")) return -1.f;
-        /* phase 4: the four launches of one layer in order, every iteration on the next layer, as
-         * inside a frame (700 MB of weights per turn: none of them is still cached when it comes
-         * round again).  A single phase launched again and again re-reads weights that partly sit
-         * in the memory-side cache and comes out faster than inside a frame. */
-        const vt_layer_dev *L = &g_vt.ac.layers[(it + 2) % TTS_HIP_AC_LAYERS];
-        int r = 0;
-        if (phase == AC_QKV || phase == 4) r |= launch_phase<AC_QKV>(L->wqkv, w.tok, L->attn_norm, w.qkv, VT_QKV_DIM);
-        if (phase == AC_WO || phase == 4) r |= launch_phase<AC_WO>(L->wo, w.qkv, NULL, w.tok, VT_DIM);
-        if (phase == AC_W13 || phase == 4) r |= launch_phase<AC_W13>(L->w13, w.tok, L->ffn_norm, w.h, 2 * VT_FFN);
-        if (phase == AC_W2 || phase == 4) r |= launch_phase<AC_W2>(L->w2, w.h, NULL, w.tok, VT_DIM);
-        if (r) return -1.f;
-    }
-    if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;
-    if (vt_check(hipEventSynchronize(g_vt.ev1), "bench sync")) return -1.f;
-    if (vt_check(hipEventElapsedTime(&ms, g_vt.ev0, g_vt.ev1), "bench time")) return -1.f;
-    return ms / (float)iters;
+    const vt_layer_dev *L = &g_vt.ac.layers[layer];
+    int r = 0;
+    if (phase == AC_QKV || phase == 4) r |= launch_phase<AC_QKV>(L->wqkv, w.tok, L->attn_norm, w.qkv, VT_QKV_DIM);
+    if (phase == AC_WO || phase == 4) r |= launch_phase<AC_WO>(L->wo, w.qkv, NULL, w.tok, VT_DIM);
+    if (phase == AC_W13 || phase == 4) r |= launch_phase<AC_W13>(L->w13, w.tok, L->ffn_norm, w.h, 2 * VT_FFN);
+    if (phase == AC_W2 || phase == 4) r |= launch_phase<AC_W2>(L->w2, w.h, NULL, w.tok, VT_DIM);
+    return r;
+}
+
+float *vt_ac_work_area(size_t *n_floats) {
+    *n_floats = AC_WORK_FLOATS;
+    return (float *)vt_scratch(sizeof(float) * AC_WORK_FLOATS);
 }
 
 /* One step boundary.  The latent ping-pongs between w->x and w->x2: `flip` counts the front

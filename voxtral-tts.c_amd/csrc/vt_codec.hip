@@ -641,36 +641,28 @@ extern "C" void tts_hip_codec_decode(const int *codes, int n_frames, float **out
     *out_n_samples = n;
 }
 
-/* Benchmarks (tts_hip_bench_kernel 20..24): average ms of one launch, events on the library's
- * stream.  0..3: the product kernel at the last stage's 1600 rows with the q|k|v, output,
- * gate|up and down matrices of layer 7, K cut as in the decoder; 4: the whole decoder on 200
- * frames of resident codes. */
-float vt_bench_codec(int which, int iters) {
-    if (!g_cd.uploaded) { vt_set_error("tts_hip_bench_kernel: codec weights not uploaded"); return -1.f; }
+/* For other translation units of the library: one launch of the decoder's product kernel at the last
+ * stage's 1600 rows with the q|k|v, output, gate|up or down matrix of layer 7 (which 0..3; K cut as in
+ * the decoder), or of the whole decoder on 200 frames of resident codes (which 4), on the decoder's own
+ * work buffers.  vt_codec_probe_buffers hands out those buffers (activations xn, att [1600, 1024] and
+ * h [1600, 4096], the codes) so that a caller can fill them. */
+int vt_codec_probe_buffers(float **xn, float **att, float **h, int **codes) {
+    if (!g_cd.uploaded) { vt_set_error("codec weights not uploaded"); return -1; }
+    if (cd_reserve(200)) { vt_set_error("codec: out of device memory"); return -1; }
+    *xn = g_cd.xn; *att = g_cd.att; *h = g_cd.h; *codes = g_cd.codes;
+    return 0;
+}
+
+int vt_codec_probe_launch(int which) {
     const int frames = 200, T = frames * 8;
-    if (cd_reserve(frames)) { vt_set_error("tts_hip_bench_kernel: out of device memory"); return -1.f; }
     const cd_layer_dev *l = &g_cd.layers[CD_LAYERS - 1];
     const float *W[4] = {l->wqkv, l->wo, l->w13, l->w2};
     const float *A[4] = {g_cd.xn, g_cd.att, g_cd.xn, g_cd.h};
     float *Cc[4] = {g_cd.part, g_cd.part, g_cd.wide, g_cd.part};
     static const int NN[4] = {3 * CD_DIM, CD_DIM, 2 * CD_HID, CD_DIM}, KK[4] = {CD_DIM, CD_DIM, CD_DIM, CD_HID};
-    if (which == 4) {
-        if (vt_check(hipMemsetAsync(g_cd.codes, 0, (size_t)frames * 37 * sizeof(int), g_vt.stream), "bench clear")) return -1.f;
-    } else {
-        /* non-zero operands: on zeros the matrix cores draw less power and run at a higher clock */
-        vt_launch_bench_fill((uint16_t *)g_cd.xn, NULL, (size_t)T * CD_DIM * 2);
-        vt_launch_bench_fill((uint16_t *)g_cd.att, NULL, (size_t)T * CD_DIM * 2);
-        vt_launch_bench_fill((uint16_t *)g_cd.h, NULL, (size_t)T * CD_HID * 2);
-    }
-    float ms = -1.f;
-    for (int it = -2; it < iters; it++) {
-        if (it == 0 && vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench start")) return -1.f;
-        if (which == 4) { if (cd_enqueue(g_cd.codes, frames, g_cd.wave)) return -1.f; }
-        else cd_gemm(Cc[which], A[which], W[which], T, NN[which], KK[which], KK[which], NN[which],
-                     which == 2 ? 1 : cd_splits(T, NN[which], KK[which]));
-    }
-    if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;
-    if (vt_check(hipEventSynchronize(g_vt.ev1), "bench sync")) return -1.f;
-    if (vt_check(hipEventElapsedTime(&ms, g_vt.ev0, g_vt.ev1), "bench time")) return -1.f;
-    return ms / (float)iters;
+    if (which == 4) return cd_enqueue(g_cd.codes, frames, g_cd.wave);
+    if (which < 0 || which > 3) return -1;
+    cd_gemm(Cc[which], A[which], W[which], T, NN[which], KK[which], KK[which], NN[which],
+            which == 2 ? 1 : cd_splits(T, NN[which], KK[which]));
+    return 0;
 }

@@ -157,7 +157,8 @@ static void free_frag(vt_layer_frag *g) {
 
 /* The fragment-order copies of a complete backbone layer (6.05 GB for 26 layers, next to the 6.05 GB of
  * the row-major ones).  A failure leaves the layer without them: the prefill then multiplies from the
- * row-major matrices with the 128 x 128 tile kernel. */
+ * row-major matrices with the 128 x 128 tile kernel, whose K cuts differ, so its results differ in the
+ * last bits from those of a context that has the copies; build_frag_or_say reports that. */
 static int build_frag(vt_layer_frag *g, const vt_layer_dev *l) {
     free_frag(g);
     struct { uint16_t **dst; const uint16_t *src; int n, k; } m[4] = {
@@ -172,6 +173,13 @@ static int build_frag(vt_layer_frag *g, const vt_layer_dev *l) {
         return -1;
     }
     return 0;
+}
+
+static void build_frag_or_say(int layer) {
+    if (build_frag(&g_vt.h_frag[layer], &g_vt.h_layers[layer]) == 0) return;
+    /* the failed allocation is already on record as an error (vt_set_error); say what follows from it */
+    fprintf(stderr, "tts_hip: layer %d has no fragment-order copy of its weights: its prefill products run from the "
+                    "row-major matrices (128 x 128 tiles, other K cuts: results differ in the last bits)\n", layer);
 }
 
 static void free_layer(vt_layer_dev *l) {
@@ -288,7 +296,7 @@ extern "C" int tts_hip_upload_llm_layer(int layer, const tts_hip_host_layer_t *s
     (void)hipStreamSynchronize(g_vt.stream);
     const int bad = upload_layer(&g_vt.h_layers[layer], src);
     if (bad) { free_layer(&g_vt.h_layers[layer]); free_frag(&g_vt.h_frag[layer]); }   /* incomplete: the backbone ends in front of it */
-    else (void)build_frag(&g_vt.h_frag[layer], &g_vt.h_layers[layer]);
+    else build_frag_or_say(layer);
     if (publish_dec_layers()) return -1;
     return bad ? -1 : 0;
 }
@@ -324,7 +332,7 @@ extern "C" int tts_hip_upload_llm_weights_n(void *decoder_ptr, int n_layers) {
             (void)publish_dec_layers();
             return -1;
         }
-        if (i < n_layers) (void)build_frag(&g_vt.h_frag[i], &g_vt.h_layers[i]);
+        if (i < n_layers) build_frag_or_say(i);
         if (i >= n_layers) { free_layer(&g_vt.h_layers[i]); free_frag(&g_vt.h_frag[i]); }   /* a shorter backbone than before */
     }
     if (publish_dec_layers()) return -1;
@@ -415,16 +423,3 @@ extern "C" void tts_hip_set_acoustic_grid(int workgroups) {
 }
 extern "C" int tts_hip_error_count(void) { return g_vt.error_count; }
 extern "C" const char *tts_hip_last_error(void) { return g_vt.last_error; }
-
-extern "C" void tts_hip_timer_start(void) {
-    (void)vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "timer start");
-}
-
-extern "C" float tts_hip_timer_stop_ms(void) {
-    float ms = -1.f;
-    if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "timer stop")) return ms;
-    if (vt_check(hipEventSynchronize(g_vt.ev1), "timer sync")) return ms;
-    (void)vt_check(hipEventElapsedTime(&ms, g_vt.ev0, g_vt.ev1), "timer elapsed");
-    if (vt_step_poll_abort()) return -1.f;      /* a step of the timed region was abandoned: no figure */
-    return ms;
-}

@@ -27,35 +27,16 @@
 
 /* Arrive at the grid barrier, request the next phase's first weight rows while
  * the other workgroups arrive, then wait. */
-#ifdef VT_TRACE
-/* Build-time instrumentation (never in the shipped library): workgroups 0 and
- * gridDim.x-1 record the 100 MHz wall clock at the points of every phase. */
-__device__ unsigned long long vt_trace_buf[2 * 4096];
-__device__ __forceinline__ void vt_tr(int &n) {
-    if (threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == gridDim.x - 1) && n < 4096)
-        vt_trace_buf[(blockIdx.x ? 4096 : 0) + n] = wall_clock64();
-    n++;
-}
-#define VT_TR(n) vt_tr(n)
-#else
-#define VT_TR(n) ((void)0)
-#endif
-
 template <class F, class W>
-__device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between, int &tn, W wait) {
-    VT_TR(tn);                      /* body done */
+__device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between, W wait) {
     vt_barrier_arrive(gs);
-    VT_TR(tn);                      /* arrived */
     between();
-    VT_TR(tn);                      /* prefetch requested */
-    const bool ok = wait();
-    VT_TR(tn);                      /* released */
-    return ok;
+    return wait();
 }
 
 template <class F>
-__device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between, int &tn) {
-    return vt_barrier_then(gs, flag, between, tn, [&] { return vt_barrier_wait(gs, flag); });
+__device__ __forceinline__ bool vt_barrier_then(vt_grid_sync &gs, int *flag, F between) {
+    return vt_barrier_then(gs, flag, between, [&] { return vt_barrier_wait(gs, flag); });
 }
 
 __global__ void __launch_bounds__(VT_STEP_THREADS)
@@ -63,7 +44,6 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
     __shared__ __attribute__((aligned(16))) float lds[VT_LDS_FLOATS];
     __shared__ int s_flag;
     u32x4 ring[VT_RING];
-    int tn = 0;
 
     if (blockIdx.x == 0)
         for (int t = (int)threadIdx.x; t < a.n_layers * VT_KV_HEADS; t += (int)blockDim.x)
@@ -95,7 +75,7 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
          * busy from the end of one phase's arithmetic to the start of the next one's */
         const bool more = l + 1 < a.n_layers;
         vt_qkv_body(ring, L, a, l, x_in, lds, [&] { vt_wo_prefetch(ring, L, VT_PART_HEAD); });
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_wo_prefetch(ring, L, VT_PART_TAIL); }, tn, wait_qkv)) return;
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_wo_prefetch(ring, L, VT_PART_TAIL); }, wait_qkv)) return;
         vt_attn_phase(a, l, lds);
         /* with 3 rows per wave the output projection leaves the ring slots from VT_WO_SLOTS on
          * free: the gate|up rows that go there are requested a phase early */
@@ -109,19 +89,19 @@ vt_decode_step_kernel(vt_step_args a, vt_grid_sync gs) {
                     vt_w13_l2_prefetch(L, att_busy);
                     if (more && vt_attn_is_direct(a)) vt_kv_l2_prefetch(a, l + 1, att_busy);
                 }
-            }, tn, wait_attn))
+            }, wait_attn))
             return;
         vt_wo_body(ring, L, a, x_in, lds, [&] { vt_w13_prefetch(ring, L, VT_PART_HEAD, 0, wo_slots); });
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L, VT_PART_TAIL, 0, wo_slots); }, tn))
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w13_prefetch(ring, L, VT_PART_TAIL, 0, wo_slots); }))
             return;
         vt_w13_body(ring, L, a, lds, [&] { vt_w2_prefetch(ring, L, VT_PART_HEAD); });
-        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w2_prefetch(ring, L, VT_PART_TAIL); }, tn)) return;
+        if (!vt_barrier_then(gs, &s_flag, [&] { vt_w2_prefetch(ring, L, VT_PART_TAIL); })) return;
         /* without a final norm the last layer's rows are the output: every workgroup writes its own and the
          * kernel ends without a last hand-over (in place is fine: the input was last read two phases ago) */
         const bool last_direct = !more && !a.final_norm;
         vt_w2_body(ring, L, a, lds, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1], VT_PART_HEAD); }, last_direct);
         if (last_direct) return;
-        if (!vt_barrier_then(gs, &s_flag, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1], VT_PART_TAIL); }, tn))
+        if (!vt_barrier_then(gs, &s_flag, [&] { if (more) vt_qkv_prefetch(ring, a.layers[l + 1], VT_PART_TAIL); }))
             return;
         x_in = a.x;
     }
@@ -187,8 +167,7 @@ vt_final_kernel(vt_step_args a) {
 /* Rows per workgroup of every phase must fit the 256-float LDS row buffer, and a lane of the
  * barrier polls VT_FLAG_LOADS flags. */
 static int grid_fits(int grid) {
-    int per = (2 * VT_FFN + grid - 1) / grid;
-    per = (per + 1) / 2 * 2;
+    const int per = vt_rows_per_wg(2 * VT_FFN, 2, grid);
     return per <= 256 && grid % VT_KV_HEADS == 0 && grid >= VT_KV_HEADS && grid <= VT_WAVE * VT_FLAG_LOADS;
 }
 
@@ -346,13 +325,6 @@ int vt_step_poll_abort(void) {
     return step_aborted(flag);
 }
 
-#ifdef VT_TRACE
-extern "C" void tts_hip_trace_read(unsigned long long *out) {
-    (void)hipDeviceSynchronize();
-    (void)hipMemcpyFromSymbol(out, HIP_SYMBOL(vt_trace_buf), sizeof(unsigned long long) * 2 * 4096);
-}
-#endif
-
 extern "C" void tts_hip_llm_forward_device(float *d_out_hidden, const float *d_input_embed, int pos) {
     if (g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_llm_forward: no weights uploaded"); return; }
     (void)vt_run_step(g_vt.d_layers, g_vt.n_dec_layers, 0, g_vt.d_dec_norm, d_input_embed,
@@ -384,7 +356,8 @@ extern "C" void tts_hip_layer_decode(int layer, float *d_hidden, int pos) {
         vt_set_error("tts_hip_layer_decode: layer %d not uploaded", layer);
         return;
     }
-    /* the step reads its input while it writes the output only at the very end,
-     * from workgroup 0, after the last barrier: in-place is safe */
+    /* in place is safe: without a final norm every workgroup writes its own rows of the output in the
+     * down projection's epilogue, and the input was last read two phases earlier (by the output
+     * projection's residual add), behind two grid-wide hand-overs */
     (void)vt_run_step(g_vt.d_layers + layer, 1, layer, NULL, d_hidden, d_hidden, pos);
 }

@@ -149,8 +149,7 @@ __device__ __forceinline__ vt_rows vt_split_rows(int n_rows, int align, int k_pe
     vt_rows r;
     const int G = (int)gridDim.x, wg = (int)blockIdx.x;
     const int nw = (int)(blockDim.x >> 6), wave = vt_wave();
-    int per_wg = (n_rows + G - 1) / G;
-    per_wg = (per_wg + align - 1) / align * align;
+    const int per_wg = vt_rows_per_wg(n_rows, align, G);
     r.wg_row0 = wg * per_wg;
     int nrows = n_rows - r.wg_row0;
     nrows = nrows < 0 ? 0 : (nrows > per_wg ? per_wg : nrows);
@@ -279,7 +278,7 @@ __device__ __forceinline__ void vt_ring_run(u32x4 (&ring)[VT_RING], const uint16
 
 /* ---- phase 1: RMSNorm + [wq;wk;wv] + RoPE + cache append ------------------ */
 
-__device__ __forceinline__ vt_rows vt_qkv_rows() { return vt_split_rows<1>(VT_QKV_DIM, 2, 0); }
+__device__ __forceinline__ vt_rows vt_qkv_rows() { return vt_split_rows<1>(VT_QKV_DIM, VT_QKV_ALIGN, 0); }
 
 __device__ __forceinline__ void vt_qkv_prefetch(u32x4 (&ring)[VT_RING], const vt_layer_dev &L,
                                                 int part = VT_PART_ALL) {
@@ -427,7 +426,8 @@ __device__ __forceinline__ void vt_attn_direct(const vt_step_args &a, int layer,
     const int wg = (int)blockIdx.x;
     const int NS = vt_attn_split(a);
     if (wg >= VT_HEADS * NS) return;
-    const int kvh = wg % VT_KV_HEADS, idx = wg / VT_KV_HEADS, head = kvh * 4 + (idx & 3), part_no = idx >> 2;
+    int kvh, head, part_no;
+    vt_attn_direct_map(wg, &kvh, &head, &part_no);
     const int nw = (int)(blockDim.x >> 6), wave = vt_wave(), lane = vt_lane();
     const int grp = lane >> 4, sub = lane & 15;
     const int slot = wave * 4 + grp, nslot = nw * 4;
@@ -480,23 +480,8 @@ __device__ __forceinline__ void vt_attn_direct(const vt_step_args &a, int layer,
 }
 
 /* The i-th of the workgroups whose q|k|v rows attention workgroup `wg` of the direct schedule reads
- * (past the last one: the first again): the owners of the 128 rows of its query head and of the new K
- * and V rows of its kv head, in the row split of vt_qkv_rows().  At most 7 + 7 + 7 on 256 workgroups. */
-__device__ __forceinline__ int vt_attn_producer(int wg, int i) {
-    const int G = (int)gridDim.x;
-    int per = (VT_QKV_DIM + G - 1) / G;
-    per = (per + 1) / 2 * 2;
-    const int kvh = wg % VT_KV_HEADS, head = kvh * 4 + ((wg / VT_KV_HEADS) & 3);
-    const int first[3] = {head * VT_HEAD_DIM, VT_Q_DIM + kvh * VT_HEAD_DIM, VT_Q_DIM + VT_KV_DIM + kvh * VT_HEAD_DIM};
-    int j = i;
-#pragma unroll
-    for (int k = 0; k < 3; k++) {
-        const int w0 = first[k] / per, n = (first[k] + VT_HEAD_DIM - 1) / per - w0 + 1;
-        if (j < n) return w0 + j;
-        j -= n;
-    }
-    return first[0] / per;
-}
+ * (vt_rowsplit.h: the same row split as vt_qkv_rows(); at most 7 + 7 + 7 on 256 workgroups). */
+__device__ __forceinline__ int vt_attn_producer(int wg, int i) { return vt_attn_producer_of((int)gridDim.x, wg, i); }
 
 /* The output projection's input vector into LDS: the attention output as it stands, or the
  * combination of the NS partials per head the split schedule left (online-softmax algebra of
@@ -759,8 +744,7 @@ __device__ __forceinline__ void vt_w13_l2_prefetch(const vt_layer_dev &L, int bu
     const int per_x = G >> 3, idle0 = busy >> 3;
     const int me = (((wg >> 3) - idle0) * (nw - 1) + vt_wave() - 1) * VT_WAVE + vt_lane();
     const int n_lanes = (per_x - idle0) * (nw - 1) * VT_WAVE;
-    int per_wg = (2 * VT_FFN + G - 1) / G;
-    per_wg = (per_wg + 1) / 2 * 2;
+    const int per_wg = vt_rows_per_wg(2 * VT_FFN, 2, G);
     const int per_wave = (per_wg + nw - 1) / nw;
     const int lines_per_row = VT_DIM * 2 / 128;
     const int total = per_x * nw * VT_L2_ROWS * lines_per_row;

@@ -9,6 +9,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "vt_rowsplit.h"
+
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -16,15 +18,6 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 
 #define VT_WAVE 64
 
-/* Model dimensions of the backbone / acoustic transformer layer. */
-#define VT_DIM      3072
-#define VT_HEADS    32
-#define VT_KV_HEADS 8
-#define VT_HEAD_DIM 128
-#define VT_Q_DIM    4096
-#define VT_KV_DIM   1024
-#define VT_QKV_DIM  6144
-#define VT_FFN      9216
 #define VT_EPS      1e-5f
 
 /* The thread index goes through an empty asm: what a phase of a persistent kernel derives from
@@ -200,8 +193,16 @@ struct vt_grid_sync {
 #define VT_POLL_SLEEP 4
 #endif
 
+/* A fence for the compiler only (no instruction): memory accesses written on one side of it are not
+ * moved to the other.  The hardware order comes from the wait for the store acknowledgements; this
+ * keeps the compiler from placing a hand-over store behind that wait, or a load of handed-over data
+ * in front of the poll that releases it. */
+__device__ __forceinline__ void vt_compiler_fence() { __atomic_signal_fence(__ATOMIC_SEQ_CST); }
+
 __device__ __forceinline__ void vt_barrier_arrive(vt_grid_sync &gs) {
+    vt_compiler_fence();
     __builtin_amdgcn_s_waitcnt(0x0F70);          /* vmcnt(0): this wave's stores are acknowledged */
+    vt_compiler_fence();
     __syncthreads();
     if (threadIdx.x < VT_FLAG_COPIES) vt_stc_u32(gs.flags + threadIdx.x * VT_FLAG_STRIDE + blockIdx.x * VT_FLAG_PAD, gs.epoch);
 }
@@ -257,6 +258,7 @@ __device__ __forceinline__ bool vt_barrier_wait_on(vt_grid_sync &gs, int *lds_fl
         if (threadIdx.x == 0) *lds_flag = ok;
     }
     __syncthreads();
+    vt_compiler_fence();                         /* loads of handed-over data stay behind the release */
     gs.epoch += 1u;
     return *lds_flag != 0;
 }

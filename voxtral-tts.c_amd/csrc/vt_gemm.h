@@ -41,8 +41,6 @@ void vt_launch_residual_norm_split(float *d_x, const float *d_part, int splits, 
 /* n_out a multiple of 4, tail_col0 of 8: planes of silu(gate)*up from interleaved (gate, up) pairs */
 void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, size_t n_out, int tail_col0,
                             const float *d_tail, int tail_planes, size_t tail_stride);
-/* benchmark input: n pseudo-random bf16 values per plane (d_lo may be NULL) */
-void vt_launch_bench_fill(uint16_t *d_hi, uint16_t *d_lo, size_t n);
 void vt_launch_sum_planes(float *d_out, const float *d_part, int splits, size_t stride, size_t n);
 
 #endif /* VT_GEMM_H */

@@ -672,20 +672,3 @@ void vt_launch_sum_planes(float *d_out, const float *d_part, int splits, size_t 
     hipLaunchKernelGGL(vt_sum_planes_kernel, dim3(gm_blocks(n)), dim3(256), 0, g_vt.stream, d_out, d_part,
                        splits, stride, n);
 }
-
-/* Benchmark input: pseudo-random bf16 values of the size of normalised activations, hi in +-(2^-7 .. 2) and
- * (d_lo != NULL) lo 2^-9 of that with a mantissa of its own.  Written over a float array as 2 n halves it
- * gives floats of the same range. */
-__global__ void vt_bench_fill_kernel(uint16_t *hi, uint16_t *lo, size_t n) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
-        unsigned h = (unsigned)i * 2654435761u + 12345u;
-        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
-        /* sign, an exponent in 120..127 (2^-7 .. 1, times 1.x), 7 mantissa bits */
-        hi[i] = (uint16_t)(((h & 1u) << 15) | ((120u + ((h >> 1) & 7u)) << 7) | ((h >> 4) & 127u));
-        if (lo) lo[i] = (uint16_t)((((h >> 11) & 1u) << 15) | ((111u + ((h >> 1) & 7u)) << 7) | ((h >> 12) & 127u));
-    }
-}
-
-void vt_launch_bench_fill(uint16_t *d_hi, uint16_t *d_lo, size_t n) {
-    hipLaunchKernelGGL(vt_bench_fill_kernel, dim3(gm_blocks(n)), dim3(256), 0, g_vt.stream, d_hi, d_lo, n);
-}

@@ -252,6 +252,12 @@ static unsigned char *s_static_ptr[VT_STATIC_MAX_DEVICES];
 static unsigned char *static_scratch(void) {
     int dev = -1;
     if (vt_check(hipGetDevice(&dev), "hipGetDevice")) return NULL;
+    /* the kernels run on the library's stream, which belongs to the device the context was made on:
+     * the array's copy on any other device is not the one they could reach */
+    if (dev != g_vt.device) {
+        vt_set_error("tts_hip_linear_bf16_noalloc: current device %d is not the device of the context (%d)", dev, g_vt.device);
+        return NULL;
+    }
     if (dev < 0 || dev >= VT_STATIC_MAX_DEVICES) {
         vt_set_error("tts_hip_linear_bf16_noalloc: device %d beyond the %d this build keeps an address for", dev,
                      VT_STATIC_MAX_DEVICES);
@@ -347,26 +353,6 @@ done:
     if (tmp_x) (void)hipFree(tmp_x);
     if (tmp_y) (void)hipFree(tmp_y);
     if (tmp_W) (void)hipFree(tmp_W);
-}
-
-extern "C" float tts_hip_bench_matvec(float *d_y, const float *d_x, const uint16_t *d_W, size_t copy_stride,
-                                      int n_copies, int in_dim, int out_dim, int iters) {
-    if (!g_vt.initialized) { vt_set_error("tts_hip_bench_matvec: backend not initialised"); return -1.f; }
-    if (!d_y || !d_x || !d_W || n_copies < 1 || in_dim < 1 || out_dim < 1 || iters < 1) {
-        vt_set_error("tts_hip_bench_matvec: bad arguments");
-        return -1.f;
-    }
-    for (int i = 0; i < n_copies; i++)                                  /* warm-up: one pass over every copy */
-        vt_launch_linear(d_y, d_x, d_W + (size_t)i * copy_stride, NULL, 1, in_dim, out_dim);
-    if (vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench record")) return -1.f;
-    for (int i = 0; i < iters; i++)
-        vt_launch_linear(d_y, d_x, d_W + (size_t)(i % n_copies) * copy_stride, NULL, 1, in_dim, out_dim);
-    if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench record")) return -1.f;
-    if (vt_check(hipEventSynchronize(g_vt.ev1), "bench sync")) return -1.f;
-    if (vt_check(hipGetLastError(), "bench launch")) return -1.f;
-    float ms = -1.f;
-    if (vt_check(hipEventElapsedTime(&ms, g_vt.ev0, g_vt.ev1), "bench elapsed")) return -1.f;
-    return ms / (float)iters;
 }
 
 /* ---- RMSNorm: one workgroup per row ------------------------------------------ */

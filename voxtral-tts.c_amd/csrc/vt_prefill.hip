@@ -444,7 +444,7 @@ static size_t pa_lds_bytes(void) {
 /* Tiles of 32 keys that cover `rows` cache rows, and the tile images of one layer's K and V (a buffer of the
  * library's own that grows with the longest cache seen) */
 static int pa_tiles(int rows) { return (rows + 31) / 32; }
-static unsigned char *pa_image(int rows) {
+unsigned char *vt_pa_image(int rows) {
     const size_t bytes = (size_t)VT_KV_HEADS * pa_tiles(rows) * PA_TILE_BYTES;
     if (bytes > g_vt.kv_img_bytes) {
         if (g_vt.d_kv_img) {
@@ -459,7 +459,7 @@ static unsigned char *pa_image(int rows) {
 
 /* d_qkv != NULL: rows start_pos .. start_pos + S - 1 are taken from the q|k|v product (summed, k rotated)
  * and appended to the cache d_K / d_V; otherwise all start_pos + S rows are in the cache already */
-static void pa_launch_image(unsigned char *d_img, const float *d_qkv, int planes, size_t plane_stride, float *d_K,
+void vt_pa_launch_image(unsigned char *d_img, const float *d_qkv, int planes, size_t plane_stride, float *d_K,
                             float *d_V, int S, int start_pos) {
     const int rows = start_pos + S;
     hipLaunchKernelGGL(vt_kv_image_kernel, dim3(pa_tiles(rows), VT_KV_HEADS), dim3(256), 0, g_vt.stream, d_img,
@@ -490,21 +490,17 @@ void vt_launch_prefill_attention_raw(float *d_out, uint16_t *d_hi, uint16_t *d_l
 void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
                                  int q_stride, const float *d_K, const float *d_V, int S, int start_pos,
                                  float scale) {
-    unsigned char *img = pa_image(start_pos + S);
+    unsigned char *img = vt_pa_image(start_pos + S);
     if (!img) return;
     /* (the image kernel only reads a cache that is complete) */
-    pa_launch_image(img, NULL, 0, 0, const_cast<float *>(d_K), const_cast<float *>(d_V), S, start_pos);
+    vt_pa_launch_image(img, NULL, 0, 0, const_cast<float *>(d_K), const_cast<float *>(d_V), S, start_pos);
     vt_launch_prefill_attention_raw(d_out, d_hi, d_lo, d_Q, q_stride, 1, 0, NULL, img, S, start_pos, scale);
 }
 
 /* ---- backbone prefill ------------------------------------------------------------ */
 
-#ifndef VT_W13_TAIL_CUT
-#define VT_W13_TAIL_CUT 4
-#endif
-
 /* K cuts of a product of `tiles` output tiles: one item per CU at most, `most` planes at most */
-static int vt_prefill_cuts(int tiles, int most) {
+int vt_prefill_cuts(int tiles, int most) {
     const int c = g_vt.n_cu / tiles;
     return c < 1 ? 1 : c > most ? most : c;
 }
@@ -531,7 +527,7 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
     const size_t n_plane = S * VT_FFN;                            /* bf16 elements per plane */
     const size_t bytes = sizeof(float) * (n_x + n_wide + n_part) + 2 * sizeof(uint16_t) * n_plane;
     float *x = (float *)vt_scratch(bytes);
-    unsigned char *img = pa_image(start_pos + seq_len);
+    unsigned char *img = vt_pa_image(start_pos + seq_len);
     if (!x || !img) return;
     float *wide = x + n_x, *part = wide + n_wide;
     uint16_t *hi = (uint16_t *)(part + n_part), *lo = hi + n_plane;
@@ -550,7 +546,7 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
         else vt_launch_gemm(wide, hi, lo, L->wqkv, seq_len, VT_QKV_DIM, VT_DIM, sp_qkv);
         /* k (rotated) and v into the cache and, with the earlier rows, into the attention's tile images; the
          * attention takes q from the product's planes itself */
-        pa_launch_image(img, wide, sp_qkv, S * VT_QKV_DIM, kc, vc, seq_len, start_pos);
+        vt_pa_launch_image(img, wide, sp_qkv, S * VT_QKV_DIM, kc, vc, seq_len, start_pos);
         vt_launch_prefill_attention_raw(NULL, hi, lo, wide, VT_QKV_DIM, sp_qkv, S * VT_QKV_DIM, g_vt.d_rope, img,
                                         seq_len, start_pos, VT_ATT_SCALE);
         if (frag) vt_launch_gemm_frag(part, VT_DIM, ps, hi, lo, F->wo, seq_len, VT_DIM, VT_Q_DIM, sp_wo);
@@ -592,78 +588,4 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
 
 extern "C" void tts_hip_llm_prefill(const float *embeds, int seq_len, int start_pos) {
     tts_hip_llm_prefill_out(embeds, seq_len, start_pos, NULL);
-}
-
-/* ---- single-kernel timing for benchmarks ---------------------------------------------
- * which 0..3: the matrix-core product at M = 512 with the q|k|v, output, gate/up and
- * down projection (splits as in the prefill), every launch on the next backbone layer's
- * weights; 4: the causal attention at 512 queries; 10..13: the four acoustic phase kernels,
- * every launch on the next acoustic layer; 14: the four phase launches of one acoustic layer
- * in order (the value is the time of all four).
- * Returns the average duration of one launch in ms (events on the internal stream), or
- * a negative value on error.  The activation planes (and q) hold pseudo-random values of the size of
- * normalised activations; the attention reads whatever the KV cache of layer 0 holds. */
-float vt_bench_acoustic_phase(int phase, int iters);
-
-extern "C" float tts_hip_bench_kernel(int which, int iters) {
-    if (!g_vt.initialized || iters < 1) { vt_set_error("tts_hip_bench_kernel: bad call"); return -1.f; }
-    if (which >= 10 && which <= 14) return vt_bench_acoustic_phase(which - 10, iters);
-    if (which >= 20 && which <= 24) return vt_bench_codec(which - 20, iters);
-    if (which < 0 || which > 4 || g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_bench_kernel: unknown kernel %d", which); return -1.f; }
-    const int S = 512;
-    if (which == 4 && g_vt.kv_max < S) { vt_set_error("tts_hip_bench_kernel: KV cache shorter than 512"); return -1.f; }
-    static const int NN[4] = {VT_QKV_DIM, VT_DIM, 2 * VT_FFN, VT_DIM}, KK[4] = {VT_DIM, VT_Q_DIM, VT_DIM, VT_FFN};
-    const int SP[4] = {vt_prefill_cuts(4 * (VT_QKV_DIM / 256), 4), vt_prefill_cuts(4 * (VT_DIM / 256), 8), 1,
-                       vt_prefill_cuts(4 * (VT_DIM / 256), 8)};
-    static const int RP[4] = {2, 4, 1, 4};            /* row-major weights: cuts that divide K */
-    const size_t n_out = (size_t)S * 2 * VT_FFN * 4, n_plane = (size_t)S * VT_FFN, n_q = (size_t)S * VT_Q_DIM;
-    const size_t bytes = sizeof(float) * (n_out + n_q) + 2 * sizeof(uint16_t) * n_plane;
-    unsigned char *base = (unsigned char *)vt_scratch(bytes);
-    if (!base) return -1.f;
-    if (vt_check(hipMemsetAsync(base, 0, bytes, g_vt.stream), "bench clear")) return -1.f;
-    float *out = (float *)base, *q = out + n_out;
-    uint16_t *hi = (uint16_t *)(q + n_q), *lo = hi + n_plane;
-    /* The kernels do the same work on any data, but not at the same clock: on planes of zeros the matrix
-     * cores draw less power and the products measure 5-15 % faster than inside a prefill.  The planes get
-     * values of the size a normalised activation has: hi = bf16 of a uniform value in (-2, 2), lo a value
-     * 2^-9 of that with its own mantissa. */
-    if (which < 4)
-        vt_launch_bench_fill(hi, lo, n_plane);
-    else                                              /* q: floats whose upper halves are such bf16 values */
-        vt_launch_bench_fill((uint16_t *)q, NULL, 2 * n_q);
-    /* the attention alone: the tile images of layer 0's cache are made once, in front of the loop (in a
-     * prefill the kernel that appends the new rows to the cache writes them) */
-    unsigned char *img = NULL;
-    if (which == 4) {
-        if (!(img = pa_image(S))) return -1.f;
-        pa_launch_image(img, NULL, 0, 0, g_hip.kv_cache_k_gpu, g_hip.kv_cache_v_gpu, S, 0);
-    }
-    float ms = -1.f;
-    for (int it = -2; it < iters; it++) {
-        if (it == 0 && vt_check(hipEventRecord(g_vt.ev0, g_vt.stream), "bench start")) return -1.f;
-        /* every launch takes the next layer's weights, as in a prefill: launched again and again on
-         * one layer they would be served from the memory-side cache */
-        const vt_layer_dev *L = &g_vt.h_layers[(it + 2) % g_vt.n_dec_layers];
-        const uint16_t *W[4] = {L->wqkv, L->wo, L->w13, L->w2};
-        const vt_layer_frag *F = &g_vt.h_frag[(it + 2) % g_vt.n_dec_layers];
-        const uint16_t *Wf[4] = {F->wqkv, F->wo, F->w13, F->w2};
-        const bool frag = F->wqkv && F->wo && F->w13 && F->w2;
-        if (which == 2 && frag) {                       /* as in the prefill: main part + K-cut tail */
-            const int tail = 8 * 256, main_cols = 2 * VT_FFN - tail;
-            uint16_t *h_hi = (uint16_t *)out, *h_lo = h_hi + n_plane;
-            vt_launch_gemm_frag_swiglu(h_hi, h_lo, VT_FFN, out + (size_t)S * 2 * VT_FFN, hi, lo, Wf[2], S, main_cols, tail, VT_DIM,
-                                       VT_W13_TAIL_CUT);
-        } else if (which == 2) {
-            const int tail = 16 * 128, main_cols = 2 * VT_FFN - tail;
-            vt_launch_gemm_ex(out, 2 * VT_FFN, 0, hi, lo, W[2], S, main_cols, VT_DIM, 1);
-            vt_launch_gemm_ex(out + (size_t)S * 2 * VT_FFN, tail, (size_t)S * tail, hi, lo,
-                              W[2] + (size_t)main_cols * VT_DIM, S, tail, VT_DIM, 4);
-        } else if (which < 4 && frag) vt_launch_gemm_frag(out, NN[which], (size_t)S * NN[which], hi, lo, Wf[which], S, NN[which], KK[which], SP[which]);
-        else if (which < 4) vt_launch_gemm(out, hi, lo, W[which], S, NN[which], KK[which], RP[which]);
-        else vt_launch_prefill_attention_raw(out, NULL, NULL, q, VT_Q_DIM, 1, 0, NULL, img, S, 0, VT_ATT_SCALE);
-    }
-    if (vt_check(hipEventRecord(g_vt.ev1, g_vt.stream), "bench stop")) return -1.f;
-    if (vt_check(hipEventSynchronize(g_vt.ev1), "bench sync")) return -1.f;
-    if (vt_check(hipEventElapsedTime(&ms, g_vt.ev0, g_vt.ev1), "bench time")) return -1.f;
-    return ms / (float)iters;
 }

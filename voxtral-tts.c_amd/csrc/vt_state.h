@@ -112,7 +112,21 @@ void vt_launch_prefill_attention(float *d_out, uint16_t *d_hi, uint16_t *d_lo, c
 /* the model's attention scale, 1/sqrt(head_dim), computed like the CPU path does (voxtral_tts_llm.c:189) */
 #define VT_ATT_SCALE (1.0f / sqrtf((float)VT_HEAD_DIM))
 void vt_codec_free(void);
-float vt_bench_codec(int which, int iters);
+/* single launches for the library's other translation units and its benchmark companion (vt_bench.hip) */
+int vt_codec_probe_buffers(float **xn, float **att, float **h, int **codes);
+int vt_codec_probe_launch(int which);
+int vt_ac_launch_layer_phase(int layer, int phase);
+float *vt_ac_work_area(size_t *n_floats);
+int vt_prefill_cuts(int tiles, int most);
+unsigned char *vt_pa_image(int rows);
+void vt_pa_launch_image(unsigned char *d_img, const float *d_qkv, int planes, size_t plane_stride, float *d_K,
+                        float *d_V, int S, int start_pos);
+void vt_launch_prefill_attention_raw(float *d_out, uint16_t *d_hi, uint16_t *d_lo, const float *d_Q,
+                                     int q_stride, int q_planes, size_t q_plane_stride, const float *d_rope,
+                                     const unsigned char *d_img, int S, int start_pos, float scale);
+#ifndef VT_W13_TAIL_CUT
+#define VT_W13_TAIL_CUT 4
+#endif
 int vt_step_resident(void);
 int vt_step_poll_abort(void);
 int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
