@@ -102,21 +102,21 @@ class Hip:
 
     def kv(self, n_layers=None):
         """Device KV caches as numpy [26, kv_max, 1024] (only uploaded layers are meaningful)."""
-        ctx = ctx()
+        g = ctx()
         shp = (26, self.kv_max, S.KV_DIM)
         k = np.empty(shp, np.float32)
         v = np.empty(shp, np.float32)
-        self.lib.tts_hip_to_host(k.ctypes.data, ctx.kv_cache_k_gpu, k.nbytes)
-        self.lib.tts_hip_to_host(v.ctypes.data, ctx.kv_cache_v_gpu, v.nbytes)
+        self.lib.tts_hip_to_host(k.ctypes.data, g.kv_cache_k_gpu, k.nbytes)
+        self.lib.tts_hip_to_host(v.ctypes.data, g.kv_cache_v_gpu, v.nbytes)
         return k, v
 
     def set_kv(self, k, v):
-        ctx = ctx()
+        g = ctx()
         k = np.ascontiguousarray(k, np.float32)
         v = np.ascontiguousarray(v, np.float32)
         assert k.shape == (26, self.kv_max, S.KV_DIM)
-        self.lib.tts_hip_to_device(ctx.kv_cache_k_gpu, k.ctypes.data, k.nbytes)
-        self.lib.tts_hip_to_device(ctx.kv_cache_v_gpu, v.ctypes.data, v.nbytes)
+        self.lib.tts_hip_to_device(g.kv_cache_k_gpu, k.ctypes.data, k.nbytes)
+        self.lib.tts_hip_to_device(g.kv_cache_v_gpu, v.ctypes.data, v.nbytes)
 
     # -- acoustic --------------------------------------------------------------
     def upload_acoustic(self, ac):
