@@ -58,7 +58,8 @@ class _Checkers:
             for d in (os.path.join(ROOT, "tests"), os.path.join(ROOT, "tests", "golden")):
                 if d not in sys.path:
                     sys.path.insert(0, d)
-                    import codec_cases
+            import cases
+            import codec_cases
             import codecsupport
             import vtsupport
             _Checkers._mods = {"cases": cases, "codec_cases": codec_cases, "codecsupport": codecsupport, "vt": vtsupport}
