@@ -285,6 +285,14 @@ void tts_hip_default_time_inv_freq(float *out, int half_dim);
  * resident at once runs schedule 1 instead), 1 = one kernel per phase.  Other values are an error
  * and leave the schedule as it is. */
 void tts_hip_set_decode_mode(int mode);
+/* Prefill schedule: 0 (default) = one launch per product and row pass; 1 = per layer, everything behind the
+ * attention (output projection, residual + RMSNorm, gate|up with SiLU*up, down projection, residual + next
+ * RMSNorm, next layer's q|k|v) is one persistent launch whose work items wait for each other per block of 128
+ * rows.  The results are the same, bit for bit; schedule 1 measures 3-9 % slower (its dependency waits cost
+ * more than the launch boundaries they replace) and is kept as a cross-check.  A context without the
+ * fragment-order weight copies, or a device on which the persistent grid cannot be resident, runs schedule 0.
+ * Other values are an error.  No counterpart in the reference. */
+void tts_hip_set_prefill_mode(int mode);
 /* Spin budget of one grid barrier of the whole-step kernel, in ticks of the 100 MHz wall clock
  * (0 = the default of 0.2 s).  When it runs out every workgroup leaves the kernel and the result is
  * invalid.  Entry points with host pointers (tts_hip_llm_forward, tts_hip_generate_frame) report

@@ -196,3 +196,41 @@ def test_prefill_row_counts_with_uneven_k_cuts():
     """300 rows are 3 row tiles: the output and down products then run in 7 K cuts of 5 or 4 (11 or 10)
     pairs of steps and q|k|v in 3; 650 rows (6 tiles) take 3 cuts and none."""
     _prefill_case(1, [300, 650], 960, lambda n: range(0, n, 7))
+
+
+@pytest.mark.parametrize("chunks", [[512], [64], [130, 7], [300], [1, 650]])
+def test_prefill_schedules_agree_bit_for_bit(chunks):
+    """Schedule 1 runs everything behind a layer's attention as one persistent launch whose work items
+    wait for each other per block of 128 rows; schedule 0 is one launch per product and row pass.  Same K
+    cuts, same tile walk, same sums in the same order: cache rows and residual stream must be equal bit
+    for bit, run after run (3 layers, so that the q|k|v product of the next layer inside the persistent
+    launch and the last layer without one are both walked)."""
+    layers = [S.Layer(11), S.Layer(12)]
+    norm = S.norm_weight(S.DIM, 98)
+    n_layers, kv_max = 3, sum(chunks) + 8
+    hip = H.Hip(kv_max=kv_max)
+    try:
+        hip.upload_decoder(layers, norm, n_layers)
+        outs = {}
+        for run, mode in enumerate((1, 0, 1)):
+            hip.lib.tts_hip_set_prefill_mode(mode)
+            hip.check()
+            hip.lib.tts_hip_memset(hip.pkg.ctx().kv_cache_k_gpu, 0, 26 * kv_max * S.KV_DIM * 4)
+            hip.lib.tts_hip_memset(hip.pkg.ctx().kv_cache_v_gpu, 0, 26 * kv_max * S.KV_DIM * 4)
+            hip.pos = 0
+            xs = []
+            for ci, s in enumerate(chunks):
+                print(f"prefill schedule {mode}, chunk of {s} rows at {hip.pos}", flush=True)
+                xs.append(hip.llm_prefill(S.f32_normal((s, S.DIM), 60 + ci), want_x=True))
+            gk, gv = hip.kv()
+            outs[run] = (np.concatenate(xs), gk[:n_layers].copy(), gv[:n_layers].copy())
+        for run in (1, 2):
+            for a, b, what in zip(outs[0], outs[run], ("residual stream", "k rows", "v rows")):
+                assert np.all(np.isfinite(a)), what
+                assert np.array_equal(a, b), (what, run, float(np.abs(a - b).max()))
+        hip.lib.tts_hip_set_prefill_mode(7)
+        assert b"tts_hip_set_prefill_mode" in hip.lib.tts_hip_last_error()
+        hip.err0 = hip.lib.tts_hip_error_count()
+    finally:
+        hip.lib.tts_hip_set_prefill_mode(0)
+        hip.close()

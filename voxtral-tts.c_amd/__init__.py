@@ -111,6 +111,7 @@ SIGNATURES = {
     "tts_hip_predict_velocity_cfg": (None, [vp, vp, vp, vp, C.c_float]),
     "tts_hip_acoustic_frame": (None, [vp, vp, vp, vp]),
     "tts_hip_set_decode_mode": (None, [C.c_int]),
+    "tts_hip_set_prefill_mode": (None, [C.c_int]),
     "tts_hip_error_count": (C.c_int, []),
     "tts_hip_last_error": (C.c_char_p, []),
     "tts_hip_split_planes": (C.c_int, [vp, vp, vp, C.c_size_t]),

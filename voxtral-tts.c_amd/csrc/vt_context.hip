@@ -413,6 +413,10 @@ extern "C" void tts_hip_set_decode_mode(int mode) {
     if (mode != 0 && mode != 1) { vt_set_error("tts_hip_set_decode_mode: unknown schedule %d", mode); return; }
     g_vt.decode_mode = mode;
 }
+extern "C" void tts_hip_set_prefill_mode(int mode) {
+    if (mode != 0 && mode != 1) { vt_set_error("tts_hip_set_prefill_mode: unknown schedule %d", mode); return; }
+    g_vt.prefill_mode = mode;
+}
 extern "C" void tts_hip_set_barrier_timeout(unsigned long long ticks) { g_vt.bar_timeout = ticks; }
 extern "C" void tts_hip_set_acoustic_grid(int workgroups) {
     if (workgroups < 0 || (g_vt.initialized && workgroups > g_vt.n_cu)) {

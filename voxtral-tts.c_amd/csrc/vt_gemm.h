@@ -43,4 +43,27 @@ void vt_launch_swiglu_split(uint16_t *d_hi, uint16_t *d_lo, const float *d_gu, s
                             const float *d_tail, int tail_planes, size_t tail_stride);
 void vt_launch_sum_planes(float *d_out, const float *d_part, int splits, size_t stride, size_t n);
 
+/* The products of one prefill layer behind its attention, with the row passes between them and the next
+ * layer's q|k|v product, as one persistent launch (vt_prefill_layer_kernel).  All weights in fragment order;
+ * every buffer distinct (each is written once per launch); cnt: vt_prefill_layer_counter_bytes() of zeros. */
+struct vt_prefill_layer_args {
+    int M;                                              /* rows */
+    const uint16_t *wo_f, *w13_f, *w2_f, *qkv_next_f;   /* qkv_next_f NULL: the last layer */
+    const float *ffn_norm, *next_norm;                  /* next_norm NULL: no planes behind the last residual add */
+    const uint16_t *attn_hi, *attn_lo;                  /* [M, 4096] attention output planes (in) */
+    float *x;                                           /* [M, 3072] residual stream (in place) */
+    float *part_a, *part_b;                             /* [fo][M, 3072] K-cut planes of the output / down projection */
+    uint16_t *n1_hi, *n1_lo, *n2_hi, *n2_lo;            /* [M, 3072] planes behind the two RMSNorms */
+    uint16_t *h_hi, *h_lo;                              /* [M, 9216] SiLU(gate) * up */
+    float *tail;                                        /* [VT_W13_TAIL_CUT][M, 2048] */
+    float *qkv;                                         /* [fq][M, 6144] K-cut planes of the next layer's q|k|v (out) */
+    int fo, fq;                                         /* K cuts of output / down, and of q|k|v */
+    unsigned *cnt;
+    int *abort_flag;
+    unsigned long long timeout;                         /* spin budget of one dependency wait, 100 MHz ticks */
+};
+int vt_prefill_layer_usable(int M);
+size_t vt_prefill_layer_counter_bytes(void);
+int vt_launch_prefill_layer(const vt_prefill_layer_args &a);
+
 #endif /* VT_GEMM_H */

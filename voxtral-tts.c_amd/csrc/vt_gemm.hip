@@ -209,14 +209,24 @@ struct gw_part {
 };
 struct gw_plan { gw_part part[2]; int n_parts; };
 
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int M, int K, int m_tiles) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    const int id = (int)blockIdx.x;
-  for (int pi = 0; pi < plan.n_parts; pi++) {
-    const gw_part &P = plan.part[pi];
+/* Stores of results that another workgroup of the SAME launch will read (the persistent layer kernel
+ * below): written through to memory, because every XCD has its own L2.  COH = false: plain stores (a
+ * kernel boundary makes them visible). */
+template <bool COH> __device__ __forceinline__ void gw_st_f32(float *p, float v) {
+    if (COH) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+template <bool COH> __device__ __forceinline__ void gw_st_u16(uint16_t *p, uint16_t v) {
+    if (COH) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+
+/* Item `id` of the set P (id < m_tiles * P.n_tiles * P.splits): one 128 x 256 tile over one K cut.  Returns
+ * the item's M tile. */
+template <bool COH>
+__device__ __forceinline__ int gw_run_item(const gw_part &P, int id, const uint16_t *Ahi, const uint16_t *Alo, int M,
+                                           int K, int m_tiles, unsigned char *lds) {
     const int n_tiles = P.n_tiles, ldc = P.ldc, items = m_tiles * n_tiles * P.splits;
-    if (id >= items) continue;
     float *C = P.C;
     const uint16_t *Wf = P.Wf;
     const size_t plane_stride = P.plane_stride;
@@ -384,8 +394,8 @@ vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int 
                 unsigned sh, sl;
                 vt_split_planes2(h, 0.f, sh, sl);
                 if (row < M) {
-                    P.h_hi[(size_t)row * P.ldh + hc] = (uint16_t)sh;
-                    P.h_lo[(size_t)row * P.ldh + hc] = (uint16_t)sl;
+                    gw_st_u16<COH>(P.h_hi + (size_t)row * P.ldh + hc, (uint16_t)sh);
+                    gw_st_u16<COH>(P.h_lo + (size_t)row * P.ldh + hc, (uint16_t)sl);
                 }
             }
     } else {
@@ -398,12 +408,333 @@ vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int 
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int row = mt * GW_TM + 32 * a + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-                if (row < M) Cs[(size_t)row * ldc + col] = acc[a][b][v];
+                if (row < M) gw_st_f32<COH>(Cs + (size_t)row * ldc + col, acc[a][b][v]);
             }
         }
     }
     __syncthreads();                 /* the next item refills the LDS stages */
-  }
+    return mt;
+}
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+vt_gemm_wide_kernel(gw_plan plan, const uint16_t *Ahi, const uint16_t *Alo, int M, int K, int m_tiles) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int id = (int)blockIdx.x;
+    for (int pi = 0; pi < plan.n_parts; pi++) {
+        const gw_part &P = plan.part[pi];
+        if (id < m_tiles * P.n_tiles * P.splits) (void)gw_run_item<false>(P, id, Ahi, Alo, M, K, m_tiles, lds);
+    }
+}
+
+/* ---- one layer's products as ONE persistent launch ----------------------------------------------
+ * Behind the attention, a prefill layer is a chain of four products with row passes between them
+ * (voxtral_tts_llm.c:326-366): output projection -> residual + RMSNorm -> gate|up with SiLU*up -> down
+ * projection -> residual + next layer's RMSNorm -> next layer's q|k|v.  As separate launches every link of
+ * that chain pays a dispatch, an empty device at its start and a drain at its end.  Here the whole chain
+ * is one list of work items in dependency order (tile items of the products, two-row items of the row
+ * passes); workgroup w of a grid of one workgroup per CU takes items w, w + G, w + 2G, ...  An item of
+ * M tile m (128 rows) waits until the items it reads from have counted themselves into that tile's
+ * counter (a bounded poll, as in vt_device.h), so only the rows that depend on each other wait for each
+ * other, a workgroup that is done early goes on to its next item, and nothing is dispatched in between.
+ * Items are numbered in dependency order and every workgroup takes its items in ascending order, so the
+ * lowest unfinished item can always run: the grid cannot deadlock as long as it is resident at once.
+ *
+ * Data that one item writes and another reads crosses XCDs, each with an L2 of its own: results are
+ * written through (agent-scope stores) and every buffer of the chain is written exactly once per launch,
+ * before anybody reads it, so no L2 can hold an older copy of a line and the products keep reading their
+ * operands through the cache; the row passes read past it (each value is read once anyway).
+ * The arithmetic is that of the separate launches, element for element: same K cuts, same tile walk, the
+ * same sums in the same order. */
+#define PF_MAX_TILES 64                 /* M tiles (8192 rows) */
+enum { PF_GEMM = 0, PF_NORM = 1, PF_TAIL = 2 };
+enum { PF_S_WO = 0, PF_S_NORM1, PF_S_W13, PF_S_W13T, PF_S_TAIL, PF_S_W2, PF_S_NORM2, PF_S_QKV, PF_N_STAGES };
+
+struct pf_stage {
+    int type, first, count;          /* items first .. first + count - 1 of the launch */
+    int dep[2];                      /* stages whose items of the same M tile must all be done (-1: none) */
+    /* PF_GEMM */
+    gw_part P;
+    const uint16_t *Ahi, *Alo;
+    int K;
+    /* PF_NORM: x += sum of `splits` planes; planes of rmsnorm(x) * w (w may be NULL) */
+    float *x;
+    const float *part;
+    int splits;
+    size_t part_stride;
+    const float *w;
+    uint16_t *hi, *lo;
+    /* PF_TAIL: vt_swiglu_pair_tail_kernel's arguments */
+    int ldh, h_col0, planes, tw;
+};
+
+struct pf_plan {
+    pf_stage st[PF_N_STAGES];
+    int total, M, m_tiles;
+    unsigned *cnt;                   /* [PF_N_STAGES][PF_MAX_TILES], zero at launch */
+    unsigned target[PF_N_STAGES];    /* items of a full M tile in each stage (the last tile of a row stage may have fewer: see pf_target) */
+    int *abort_flag;
+    unsigned long long timeout;
+};
+
+/* Buffer accesses with the device-scope bit (sc1): `p` is the same in every lane (it becomes the
+ * descriptor's base), the element index is per lane and stays below 2^31 bytes (the launcher checks the
+ * buffer sizes). */
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t pf_rsrc(const void *p) {
+    return __builtin_amdgcn_make_buffer_rsrc((void *)p, 0, 0x7ffffff0, 0x00020000);
+}
+__device__ __forceinline__ f32x4 pf_ldc4(const float *p, size_t idx) {
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(pf_rsrc(p), (int)(idx * 4), 0, 16 /* sc1 */);
+    return f32x4{__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+}
+__device__ __forceinline__ void pf_stc4(float *p, size_t idx, f32x4 v) {
+    const u32x4 u = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+    __builtin_amdgcn_raw_buffer_store_b128(u, pf_rsrc(p), (int)(idx * 4), 0, 16 /* sc1 */);
+}
+__device__ __forceinline__ void pf_stc2(uint16_t *p, size_t idx, u32x2 v) {
+    __builtin_amdgcn_raw_buffer_store_b64(v, pf_rsrc(p), (int)(idx * 2), 0, 16 /* sc1 */);
+}
+
+/* Items of M tile m that stage s counts: all of a tile's product items, or one per two rows of the tile */
+__device__ __forceinline__ unsigned pf_target(const pf_plan &pl, int s, int m) {
+    if (pl.st[s].type == PF_GEMM) return pl.target[s];
+    const int rows = min(GW_TM, pl.M - m * GW_TM);
+    return (unsigned)((rows + 1) / 2);
+}
+
+/* residual + RMSNorm + plane split of rows row0, row0 + 1 (vt_residual_norm_split_kernel's arithmetic, 256
+ * threads per row); all loads of both rows are requested before the first is used */
+__device__ __forceinline__ void pf_norm_rows(const pf_stage &st, int row0, int M, float *red) {
+    constexpr int NJ = VT_DIM / 1024;
+    const int t = (int)threadIdx.x;
+    f32x4 v[2][NJ], pp[2][NJ];
+    const int n_rows = min(2, M - row0);
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const size_t row = (size_t)(r < n_rows ? row0 + r : row0);
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const size_t i = row * VT_DIM + 4 * ((size_t)t + 256 * j);
+            v[r][j] = pf_ldc4(st.x, i);
+            pp[r][j] = pf_ldc4(st.part, i);
+        }
+    }
+    for (int s = 1; s < st.splits; s++) {
+        f32x4 q[2][NJ];
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const size_t row = (size_t)(r < n_rows ? row0 + r : row0);
+#pragma unroll
+            for (int j = 0; j < NJ; j++) q[r][j] = pf_ldc4(st.part + (size_t)s * st.part_stride, row * VT_DIM + 4 * ((size_t)t + 256 * j));
+        }
+#pragma unroll
+        for (int r = 0; r < 2; r++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                f32x4 &p = pp[r][j];
+                const f32x4 qq = q[r][j];
+                p.x = __fadd_rn(p.x, qq.x); p.y = __fadd_rn(p.y, qq.y); p.z = __fadd_rn(p.z, qq.z); p.w = __fadd_rn(p.w, qq.w);
+            }
+    }
+    float ss[2] = {0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 2; r++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            f32x4 a = v[r][j];
+            const f32x4 p = pp[r][j];
+            a.x = __fadd_rn(a.x, p.x); a.y = __fadd_rn(a.y, p.y); a.z = __fadd_rn(a.z, p.z); a.w = __fadd_rn(a.w, p.w);
+            v[r][j] = a;
+            if (r < n_rows) pf_stc4(st.x, (size_t)(row0 + r) * VT_DIM + 4 * ((size_t)t + 256 * j), a);
+            ss[r] = fmaf(a.x, a.x, ss[r]); ss[r] = fmaf(a.y, a.y, ss[r]);
+            ss[r] = fmaf(a.z, a.z, ss[r]); ss[r] = fmaf(a.w, a.w, ss[r]);
+        }
+    if (!st.w) return;
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const float w_sum = vt_wave_sum(ss[r]);
+        if (vt_lane() == 0) red[4 * r + vt_wave()] = w_sum;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const float tot = (red[4 * r] + red[4 * r + 1]) + (red[4 * r + 2] + red[4 * r + 3]);
+        const float inv = 1.0f / sqrtf(tot / (float)VT_DIM + VT_EPS);
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const int c = 4 * (t + 256 * j);
+            const f32x4 g = *reinterpret_cast<const f32x4 *>(st.w + c);
+            u32x2 sph, spl;
+            vt_split_planes4(__fmul_rn(__fmul_rn(v[r][j].x, inv), g.x), __fmul_rn(__fmul_rn(v[r][j].y, inv), g.y),
+                             __fmul_rn(__fmul_rn(v[r][j].z, inv), g.z), __fmul_rn(__fmul_rn(v[r][j].w, inv), g.w), sph, spl);
+            if (r < n_rows) {
+                pf_stc2(st.hi, (size_t)(row0 + r) * VT_DIM + c, sph);
+                pf_stc2(st.lo, (size_t)(row0 + r) * VT_DIM + c, spl);
+            }
+        }
+    }
+    __syncthreads();                 /* red is free again */
+}
+
+/* the K-cut tail of the paired gate|up product for rows row0, row0 + 1 (vt_swiglu_pair_tail_kernel's arithmetic;
+ * tw / 8 threads per row, tw <= 2048) */
+__device__ __forceinline__ void pf_tail_rows(const pf_stage &st, int row0, int M) {
+    const int per_row = st.tw / 8, q = (int)threadIdx.x;
+    if (q >= per_row) return;
+    const int blk = q >> 3, c = (q & 7) * 4;
+    const size_t stride = st.part_stride;
+    for (int r = 0; r < 2 && row0 + r < M; r++) {
+        const size_t at_in = (size_t)(row0 + r) * st.tw + 64 * blk + c;
+        f32x4 g = pf_ldc4(st.part, at_in), u = pf_ldc4(st.part, at_in + 32);
+        for (int p = 1; p < st.planes; p++) {
+            const f32x4 g2 = pf_ldc4(st.part + p * stride, at_in), u2 = pf_ldc4(st.part + p * stride, at_in + 32);
+            g.x = __fadd_rn(g.x, g2.x); g.y = __fadd_rn(g.y, g2.y); g.z = __fadd_rn(g.z, g2.z); g.w = __fadd_rn(g.w, g2.w);
+            u.x = __fadd_rn(u.x, u2.x); u.y = __fadd_rn(u.y, u2.y); u.z = __fadd_rn(u.z, u2.z); u.w = __fadd_rn(u.w, u2.w);
+        }
+        const float a = __fmul_rn(__fdiv_rn(g.x, __fadd_rn(1.0f, expf(-g.x))), u.x);
+        const float b = __fmul_rn(__fdiv_rn(g.y, __fadd_rn(1.0f, expf(-g.y))), u.y);
+        const float cc = __fmul_rn(__fdiv_rn(g.z, __fadd_rn(1.0f, expf(-g.z))), u.z);
+        const float d = __fmul_rn(__fdiv_rn(g.w, __fadd_rn(1.0f, expf(-g.w))), u.w);
+        u32x2 sph, spl;
+        vt_split_planes4(a, b, cc, d, sph, spl);
+        const size_t at = (size_t)(row0 + r) * st.ldh + st.h_col0 + 32 * blk + c;
+        pf_stc2(st.hi, at, sph);
+        pf_stc2(st.lo, at, spl);
+    }
+}
+
+/* Waits until stage `dep` has counted all its items of M tile m; false when the spin budget ran out or
+ * another workgroup has given up (then everybody leaves the kernel). */
+__device__ __forceinline__ bool pf_wait(const pf_plan &pl, int dep, int m, int *lds_ok) {
+    if (threadIdx.x < VT_WAVE) {
+        const unsigned want = pf_target(pl, dep, m);
+        const unsigned *c = pl.cnt + dep * PF_MAX_TILES + m;
+        const unsigned long long t0 = wall_clock64();
+        int ok = 1;
+        while (__hip_atomic_load(c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
+            if (__hip_atomic_load(pl.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0 ||
+                wall_clock64() - t0 > pl.timeout) {
+                ok = 0;
+                break;
+            }
+            __builtin_amdgcn_s_sleep(8);
+        }
+        if (!ok && threadIdx.x == 0) __hip_atomic_store(pl.abort_flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0) *lds_ok = ok;
+    }
+    __syncthreads();
+    vt_compiler_fence();
+    return *lds_ok != 0;
+}
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+vt_prefill_layer_kernel(pf_plan pl) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    __shared__ float s_red[8];
+    __shared__ int s_ok;
+    for (int g = (int)blockIdx.x; g < pl.total; g += (int)gridDim.x) {
+        int s = 0;
+        while (s + 1 < PF_N_STAGES && g >= pl.st[s].first + pl.st[s].count) s++;
+        const pf_stage &st = pl.st[s];
+        const int i = g - st.first;
+        int m;
+        if (st.type == PF_GEMM) {
+            /* the M tile of item i, as gw_run_item maps it */
+            const int items = st.count;
+            const int li = (items & 7) == 0 ? (i & 7) * (items >> 3) + (i >> 3) : i;
+            m = li % pl.m_tiles;
+        } else {
+            m = (2 * i) / GW_TM;
+        }
+        for (int d = 0; d < 2; d++)
+            if (st.dep[d] >= 0 && !pf_wait(pl, st.dep[d], m, &s_ok)) return;
+        if (st.type == PF_GEMM) (void)gw_run_item<true>(st.P, i, st.Ahi, st.Alo, pl.M, st.K, pl.m_tiles, lds);
+        else if (st.type == PF_NORM) pf_norm_rows(st, 2 * i, pl.M, s_red);
+        else pf_tail_rows(st, 2 * i, pl.M);
+        /* this item's results are in memory before it counts itself in */
+        vt_compiler_fence();
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        vt_compiler_fence();
+        __syncthreads();
+        if (threadIdx.x == 0)
+            __hip_atomic_fetch_add(pl.cnt + s * PF_MAX_TILES + m, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+static int pf_ready(void) {
+    static int state = 0;                /* 0 not asked, 1 usable, -1 not */
+    if (state) return state > 0;
+    state = -1;
+    if (hipFuncSetAttribute((const void *)vt_prefill_layer_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, GW_LDS) !=
+        hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    /* the item counters need every workgroup of the grid on the device at once */
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, vt_prefill_layer_kernel, 256, GW_LDS) != hipSuccess) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    if (per_cu >= 1) state = 1;
+    return state > 0;
+}
+
+int vt_prefill_layer_usable(int M) {
+    /* the sc1 accesses take 32-bit byte offsets: the largest buffer (the K-cut planes) stays below 2 GiB */
+    return M >= 1 && (M + GW_TM - 1) / GW_TM <= PF_MAX_TILES && (size_t)M * VT_FFN * 4 < ((size_t)1 << 31) && pf_ready();
+}
+
+size_t vt_prefill_layer_counter_bytes(void) { return sizeof(unsigned) * PF_N_STAGES * PF_MAX_TILES; }
+
+int vt_launch_prefill_layer(const vt_prefill_layer_args &a) {
+    if (!vt_prefill_layer_usable(a.M)) { vt_set_error("prefill layer kernel: not usable for %d rows", a.M); return -1; }
+    const int M = a.M, m_tiles = (M + GW_TM - 1) / GW_TM;
+    const bool tail = m_tiles == 4;      /* 4 x 72 gate|up tiles on 256 CUs: the last 8 N tiles get their K cut (as vt_launch_gemm_frag_swiglu's callers do) */
+    const int n_tail = tail ? 8 * GW_TN : 0, n_main = 2 * VT_FFN - n_tail;
+    const size_t ps = (size_t)M * VT_DIM;
+    pf_plan pl = {};
+    pl.M = M;
+    pl.m_tiles = m_tiles;
+    pl.cnt = a.cnt;
+    pl.abort_flag = a.abort_flag;
+    pl.timeout = a.timeout;
+    for (int s = 0; s < PF_N_STAGES; s++) { pl.st[s].dep[0] = pl.st[s].dep[1] = -1; pl.st[s].type = PF_GEMM; }
+    auto gemm = [&](int s, float *C, const uint16_t *Wf, size_t plane_stride, int ldc, int N, int splits, int K,
+                    const uint16_t *Ahi, const uint16_t *Alo, uint16_t *h_hi, uint16_t *h_lo, int dep0, int dep1) {
+        pf_stage &st = pl.st[s];
+        st.type = PF_GEMM;
+        st.P = gw_part{C, Wf, plane_stride, ldc, N / GW_TN, splits, K / (2 * GM_BK), h_hi, h_lo, VT_FFN, 0};
+        st.Ahi = Ahi; st.Alo = Alo; st.K = K;
+        st.count = Wf ? m_tiles * (N / GW_TN) * splits : 0;
+        st.dep[0] = dep0; st.dep[1] = dep1;
+        pl.target[s] = (unsigned)((N / GW_TN) * splits);
+    };
+    auto rows = [&](int s, int type, int dep0, bool present) {
+        pf_stage &st = pl.st[s];
+        st.type = type;
+        st.count = present ? (M + 1) / 2 : 0;
+        st.dep[0] = dep0;
+    };
+    gemm(PF_S_WO, a.part_a, a.wo_f, ps, VT_DIM, VT_DIM, a.fo, VT_Q_DIM, a.attn_hi, a.attn_lo, NULL, NULL, -1, -1);
+    rows(PF_S_NORM1, PF_NORM, PF_S_WO, true);
+    { pf_stage &st = pl.st[PF_S_NORM1]; st.x = a.x; st.part = a.part_a; st.splits = a.fo; st.part_stride = ps; st.w = a.ffn_norm; st.hi = a.n1_hi; st.lo = a.n1_lo; }
+    gemm(PF_S_W13, NULL, a.w13_f, 0, 0, n_main, 1, VT_DIM, a.n1_hi, a.n1_lo, a.h_hi, a.h_lo, PF_S_NORM1, -1);
+    gemm(PF_S_W13T, a.tail, tail ? a.w13_f + (size_t)n_main * VT_DIM : NULL, (size_t)M * n_tail, n_tail, tail ? n_tail : GW_TN,
+         VT_W13_TAIL_CUT, VT_DIM, a.n1_hi, a.n1_lo, NULL, NULL, PF_S_NORM1, -1);
+    rows(PF_S_TAIL, PF_TAIL, PF_S_W13T, tail);
+    { pf_stage &st = pl.st[PF_S_TAIL]; st.part = a.tail; st.planes = VT_W13_TAIL_CUT; st.part_stride = (size_t)M * n_tail; st.tw = n_tail;
+      st.ldh = VT_FFN; st.h_col0 = n_main / 2; st.hi = a.h_hi; st.lo = a.h_lo; }
+    gemm(PF_S_W2, a.part_b, a.w2_f, ps, VT_DIM, VT_DIM, a.fo, VT_FFN, a.h_hi, a.h_lo, NULL, NULL, PF_S_W13, tail ? PF_S_TAIL : -1);
+    rows(PF_S_NORM2, PF_NORM, PF_S_W2, true);
+    { pf_stage &st = pl.st[PF_S_NORM2]; st.x = a.x; st.part = a.part_b; st.splits = a.fo; st.part_stride = ps; st.w = a.next_norm; st.hi = a.n2_hi; st.lo = a.n2_lo; }
+    gemm(PF_S_QKV, a.qkv, a.qkv_next_f, (size_t)M * VT_QKV_DIM, VT_QKV_DIM, VT_QKV_DIM, a.fq, VT_DIM, a.n2_hi, a.n2_lo, NULL, NULL,
+         PF_S_NORM2, -1);
+    int first = 0;
+    for (int s = 0; s < PF_N_STAGES; s++) { pl.st[s].first = first; first += pl.st[s].count; }
+    pl.total = first;
+    const int grid = g_vt.n_cu < pl.total ? g_vt.n_cu : pl.total;
+    hipLaunchKernelGGL(vt_prefill_layer_kernel, dim3(grid), dim3(256), GW_LDS, g_vt.stream, pl);
+    return vt_check(hipGetLastError(), "prefill layer launch");
 }
 
 static int gm_blocks(size_t n);

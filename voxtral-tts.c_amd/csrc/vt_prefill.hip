@@ -505,6 +505,77 @@ int vt_prefill_cuts(int tiles, int most) {
     return c < 1 ? 1 : c > most ? most : c;
 }
 
+/* The prefill with one persistent launch per layer for everything behind the attention
+ * (vt_prefill_layer_kernel): per layer the k|v kernel, the attention and that launch, which also multiplies
+ * the next layer's q|k|v.  Same arithmetic as the launch-per-product schedule below, bit for bit.
+ * Measured slower than that schedule at every length (512 rows: 8.29 against 7.65 ms on the same box; 64 rows
+ * 4.53 / 4.34; 2048 rows 29.96 / 29.77): a dependency wait costs about 5 us (results written through and
+ * acknowledged, counter, poll, first operand loads from memory) against about 1.5 us for a launch boundary,
+ * and with one item per workgroup and stage there is nothing to overlap it with (the same kernel with the
+ * waits taken out, results wrong, takes 7.34 ms).  It is therefore the optional schedule, not the default. */
+static void prefill_persistent(const float *embeds, int seq_len, int start_pos, float *out_x) {
+    const size_t S = (size_t)seq_len;
+    hipStream_t st = g_vt.stream;
+    const int m_tiles = (seq_len + 127) / 128, n_layers = g_vt.n_dec_layers;
+    const int fq = vt_prefill_cuts(m_tiles * (VT_QKV_DIM / 256), 4), fo = vt_prefill_cuts(m_tiles * (VT_DIM / 256), 8);
+    /* work area: x | q|k|v planes | two sets of K-cut planes | gate|up tail planes | counters | bf16 planes */
+    const size_t n_x = S * VT_DIM, n_wide = S * 4 * VT_QKV_DIM, n_part = 8 * S * VT_DIM, n_tail = (size_t)VT_W13_TAIL_CUT * S * 2048;
+    const size_t cnt_bytes = vt_prefill_layer_counter_bytes() * n_layers;
+    const size_t n_p3 = S * VT_DIM, n_p4 = S * VT_Q_DIM, n_p9 = S * VT_FFN;     /* bf16 elements per plane */
+    const size_t bytes = sizeof(float) * (n_x + n_wide + 2 * n_part + n_tail) + cnt_bytes +
+                         2 * sizeof(uint16_t) * (2 * n_p3 + n_p4 + n_p9);
+    float *x = (float *)vt_scratch(bytes);
+    unsigned char *img = vt_pa_image(start_pos + seq_len);
+    if (!x || !img) return;
+    float *wide = x + n_x, *part_a = wide + n_wide, *part_b = part_a + n_part, *tail = part_b + n_part;
+    unsigned *cnt = (unsigned *)(tail + n_tail);
+    uint16_t *n1_hi = (uint16_t *)((unsigned char *)cnt + cnt_bytes), *n1_lo = n1_hi + n_p3;
+    uint16_t *n2_hi = n1_lo + n_p3, *n2_lo = n2_hi + n_p3;
+    uint16_t *at_hi = n2_lo + n_p3, *at_lo = at_hi + n_p4;
+    uint16_t *h_hi = at_lo + n_p4, *h_lo = h_hi + n_p9;
+    int *abort_flag = g_vt.d_abort + 8;
+
+    VT_TRYV(hipMemcpyAsync(x, embeds, sizeof(float) * n_x, hipMemcpyDefault, st));
+    VT_TRYV(hipMemsetAsync(cnt, 0, cnt_bytes, st));
+    vt_launch_residual_norm_split(x, NULL, 0, 0, g_vt.h_layers[0].attn_norm, n2_hi, n2_lo, seq_len);
+    vt_launch_gemm_frag(wide, VT_QKV_DIM, S * VT_QKV_DIM, n2_hi, n2_lo, g_vt.h_frag[0].wqkv, seq_len, VT_QKV_DIM, VT_DIM, fq);
+    for (int l = 0; l < n_layers; l++) {
+        const vt_layer_dev *L = &g_vt.h_layers[l];
+        const vt_layer_frag *F = &g_vt.h_frag[l];
+        float *kc = g_hip.kv_cache_k_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
+        float *vc = g_hip.kv_cache_v_gpu + (size_t)l * g_vt.kv_max * VT_KV_DIM;
+        vt_pa_launch_image(img, wide, fq, S * VT_QKV_DIM, kc, vc, seq_len, start_pos);
+        vt_launch_prefill_attention_raw(NULL, at_hi, at_lo, wide, VT_QKV_DIM, fq, S * VT_QKV_DIM, g_vt.d_rope, img,
+                                        seq_len, start_pos, VT_ATT_SCALE);
+        const bool more = l + 1 < n_layers;
+        vt_prefill_layer_args a = {};
+        a.M = seq_len;
+        a.wo_f = F->wo; a.w13_f = F->w13; a.w2_f = F->w2;
+        a.qkv_next_f = more ? g_vt.h_frag[l + 1].wqkv : NULL;
+        a.ffn_norm = L->ffn_norm;
+        a.next_norm = more ? g_vt.h_layers[l + 1].attn_norm : NULL;
+        a.attn_hi = at_hi; a.attn_lo = at_lo;
+        a.x = x; a.part_a = part_a; a.part_b = part_b;
+        a.n1_hi = n1_hi; a.n1_lo = n1_lo; a.n2_hi = n2_hi; a.n2_lo = n2_lo;
+        a.h_hi = h_hi; a.h_lo = h_lo; a.tail = tail; a.qkv = wide;
+        a.fo = fo; a.fq = fq;
+        a.cnt = cnt + (size_t)l * (vt_prefill_layer_counter_bytes() / sizeof(unsigned));
+        a.abort_flag = abort_flag;
+        a.timeout = g_vt.bar_timeout ? g_vt.bar_timeout : 200000000ull;      /* default 2 s of the 100 MHz wall clock */
+        if (vt_launch_prefill_layer(a)) return;
+    }
+    VT_TRYV(hipGetLastError());
+    VT_TRYV(hipStreamSynchronize(st));
+    int gave_up = 0;
+    VT_TRYV(hipMemcpy(&gave_up, abort_flag, sizeof gave_up, hipMemcpyDeviceToHost));
+    if (gave_up) {
+        (void)hipMemset(abort_flag, 0, sizeof(int));
+        vt_set_error("tts_hip_llm_prefill: a dependency wait of the layer kernel timed out; the kernel left early, result invalid");
+        return;
+    }
+    if (out_x) VT_TRYV(hipMemcpy(out_x, x, sizeof(float) * n_x, hipMemcpyDefault));
+}
+
 extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int start_pos, float *out_x) {
     if (!g_vt.initialized || g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_llm_prefill: no weights uploaded"); return; }
     if (seq_len < 1 || start_pos < 0 || start_pos + seq_len > g_vt.kv_max) {
@@ -514,6 +585,17 @@ extern "C" void tts_hip_llm_prefill_out(const float *embeds, int seq_len, int st
     }
     const size_t S = (size_t)seq_len;
     hipStream_t st = g_vt.stream;
+    {
+        bool all_frag = true;
+        for (int l = 0; l < g_vt.n_dec_layers; l++) {
+            const vt_layer_frag *F = &g_vt.h_frag[l];
+            all_frag = all_frag && F->wqkv && F->wo && F->w13 && F->w2;
+        }
+        if (g_vt.prefill_mode == 1 && all_frag && vt_prefill_layer_usable(seq_len)) {
+            prefill_persistent(embeds, seq_len, start_pos, out_x);
+            return;
+        }
+    }
     /* work area: x | wide f32 (qkv or gate/up) | q | partial planes | hi | lo */
     /* K is cut into as many ranges as give every CU at most one item (M tiles x N tiles x cuts; the cuts
      * need not divide K): 4 M tiles at 512 rows are 96 / 48 / 48 tiles for q|k|v / output / down, i.e.

@@ -51,6 +51,7 @@ struct vt_state {
     hipStream_t stream;
     hipEvent_t ev0, ev1;
     int decode_mode;
+    int prefill_mode;             /* 0 = one launch per product and row pass, 1 = one persistent launch per layer behind the attention */
 
     /* backbone weights */
     vt_layer_dev h_layers[TTS_HIP_DEC_LAYERS];
