@@ -325,6 +325,9 @@ int vt_step_poll_abort(void) {
     return step_aborted(flag);
 }
 
+/* The same for a caller that has already read the abort flag and found it set. */
+int vt_step_poll_abort_now(void) { return step_aborted(1); }
+
 extern "C" void tts_hip_llm_forward_device(float *d_out_hidden, const float *d_input_embed, int pos) {
     if (g_vt.n_dec_layers < 1) { vt_set_error("tts_hip_llm_forward: no weights uploaded"); return; }
     (void)vt_run_step(g_vt.d_layers, g_vt.n_dec_layers, 0, g_vt.d_dec_norm, d_input_embed,

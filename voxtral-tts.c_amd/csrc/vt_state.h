@@ -130,6 +130,7 @@ void vt_launch_prefill_attention_raw(float *d_out, uint16_t *d_hi, uint16_t *d_l
 #endif
 int vt_step_resident(void);
 int vt_step_poll_abort(void);
+int vt_step_poll_abort_now(void);
 int vt_run_step(const vt_layer_dev *d_layers, int n_layers, int first_layer,
                 const float *d_final_norm, const float *d_in, float *d_out, int pos);
 
