@@ -289,6 +289,7 @@ def bench_prefill(args):
     hip.upload_decoder(layers, final_norm, N_LAYERS)
     t_up = time.time() - t0
     d_e = H.DevBuf.from_numpy(lib, embeds)
+    lib.tts_hip_set_prefill_mode(args.prefill_mode)
     for _ in range(W):
         lib.tts_hip_llm_prefill(d_e.ptr, PREFILL_LEN, 0)
     lib.tts_hip_sync()
@@ -318,7 +319,8 @@ def bench_prefill(args):
         "data": "synthetic",
         "config": {"workload": "26-layer backbone prefill of 512 random token ids, causal GQA attention "
                                "(BASELINE.json configs[3])",
-                   "layers": N_LAYERS, "seq_len": PREFILL_LEN, "weights": "bf16 N(0,0.02) seeded, truncated"},
+                   "layers": N_LAYERS, "seq_len": PREFILL_LEN, "weights": "bf16 N(0,0.02) seeded, truncated",
+                   "schedule": ("one launch per product and row pass", "one persistent launch per layer behind the attention")[args.prefill_mode]},
         "tokens_per_s": round(PREFILL_LEN / (ms_step * 1e-3), 1),
         "tflops": round((gemm_fl + attn_fl) / ms_step / 1e9, 1),
         "roofline": {
@@ -1000,6 +1002,8 @@ def main():
     ap.add_argument("--workload", choices=("decode", "prefill", "acoustic", "frame", "codec", "matvec", "layer"), default="decode",
                     help="decode = the headline metric; prefill / acoustic = the other two configurations")
     ap.add_argument("--mode", type=int, default=0, choices=(0, 1), help="0 persistent kernel, 1 per-phase kernels")
+    ap.add_argument("--prefill-mode", type=int, default=0, choices=(0, 1),
+                    help="--workload prefill: 0 one launch per product and row pass, 1 one persistent launch per layer")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--no-workloads", action="store_true",
                     help="leave the short runs of the other configurations out of the default line")
