@@ -56,36 +56,43 @@
 #define CG_BN 128
 #define CG_BK 32
 #define CG_PITCH 36
+#ifndef CG_W64
+#define CG_W64 2            /* waves per SIMD the 64-row kernel is compiled for */
+#endif
 
 typedef float cd_f16v __attribute__((ext_vector_type(16)));
 
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2)))
-vt_codec_gemm_kernel(float *__restrict__ C, const float *__restrict__ A, const float *__restrict__ W,
-                     int M, int N, int K, int lda, int ldc, size_t plane_stride) {
-    __shared__ float As[CG_BM * CG_PITCH];
+template <int BM>
+__device__ __forceinline__ void cd_gemm_tile(float *__restrict__ C, const float *__restrict__ A, const float *__restrict__ W,
+                                             int M, int N, int K, int lda, int ldc, size_t plane_stride) {
+    constexpr int MI = BM / 64;              /* 32-row blocks per wave */
+    constexpr int AP = BM / 32;              /* staging passes of the activation tile */
+    __shared__ float As[BM * CG_PITCH];
     __shared__ float Ws[CG_BN * CG_PITCH];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * CG_BM, n0 = blockIdx.x * CG_BN;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * CG_BN;
     const int kper = K / gridDim.z, kbeg = blockIdx.z * kper;
 
     /* staging: 4 passes of 32 rows for each operand, 16 bytes per thread and pass */
     const int lr = tid >> 3, lc = (tid & 7) * 4;
-    const float *ap[4], *wp[4];
+    const float *ap[AP], *wp[4];
 #pragma unroll
     for (int p = 0; p < 4; p++) {
-        int am = m0 + p * 32 + lr;
-        am = am < M ? am : M - 1;
-        ap[p] = A + (size_t)am * lda + kbeg + lc;
+        if (p < AP) {
+            int am = m0 + p * 32 + lr;
+            am = am < M ? am : M - 1;
+            ap[p] = A + (size_t)am * lda + kbeg + lc;
+        }
         wp[p] = W + (size_t)(n0 + p * 32 + lr) * K + kbeg + lc;
     }
-    f32x4 ra[4], rw[4];       /* clang vectors: HIP's float4 structs in an array end up in LDS, not registers */
+    f32x4 ra[AP], rw[4];      /* clang vectors: HIP's float4 structs in an array end up in LDS, not registers */
 #pragma unroll
-    for (int p = 0; p < 4; p++) { ra[p] = *(const f32x4 *)ap[p]; rw[p] = *(const f32x4 *)wp[p]; }
+    for (int p = 0; p < 4; p++) { if (p < AP) ra[p] = *(const f32x4 *)ap[p]; rw[p] = *(const f32x4 *)wp[p]; }
 
-    cd_f16v acc[2][2];
+    cd_f16v acc[MI][2];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -96,7 +103,7 @@ vt_codec_gemm_kernel(float *__restrict__ C, const float *__restrict__ A, const f
         __syncthreads();
 #pragma unroll
         for (int p = 0; p < 4; p++) {
-            *(f32x4 *)&As[(p * 32 + lr) * CG_PITCH + lc] = ra[p];
+            if (p < AP) *(f32x4 *)&As[(p * 32 + lr) * CG_PITCH + lc] = ra[p];
             *(f32x4 *)&Ws[(p * 32 + lr) * CG_PITCH + lc] = rw[p];
         }
         __syncthreads();
@@ -107,21 +114,21 @@ vt_codec_gemm_kernel(float *__restrict__ C, const float *__restrict__ A, const f
             const int kn = k0 + CG_BK < kper ? k0 + CG_BK : k0;
 #pragma unroll
             for (int p = 0; p < 4; p++) {
-                ra[p] = *(const f32x4 *)(ap[p] + kn);
+                if (p < AP) ra[p] = *(const f32x4 *)(ap[p] + kn);
                 rw[p] = *(const f32x4 *)(wp[p] + kn);
             }
             __builtin_amdgcn_sched_barrier(0);          /* requests first, products behind them */
         }
 #pragma unroll
         for (int kg = 0; kg < CG_BK; kg += 8) {
-            f32x4 fa[2], fw[2];
+            f32x4 fa[MI], fw[2];
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                fa[i] = *(const f32x4 *)&As[(wm * 64 + i * 32 + fr) * CG_PITCH + kg + fk];
+                if (i < MI) fa[i] = *(const f32x4 *)&As[(wm * (BM / 2) + i * 32 + fr) * CG_PITCH + kg + fk];
                 fw[i] = *(const f32x4 *)&Ws[(wn * 64 + i * 32 + fr) * CG_PITCH + kg + fk];
             }
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < MI; i++)
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i].x, fw[j].x, acc[i][j], 0, 0, 0);
@@ -134,16 +141,31 @@ vt_codec_gemm_kernel(float *__restrict__ C, const float *__restrict__ A, const f
     /* accumulator element v of a lane: column lane % 32, row 8 * (v / 4) + 4 * (lane / 32) + v % 4 */
     float *Cp = C + (size_t)blockIdx.z * plane_stride;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MI; i++)
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int n = n0 + wn * 64 + j * 32 + (lane & 31);
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int m = m0 + wm * 64 + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
+                const int m = m0 + wm * (BM / 2) + i * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
                 if (m < M && n < N) Cp[(size_t)m * ldc + n] = acc[i][j][v];
             }
         }
+}
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2)))
+vt_codec_gemm_kernel(float *__restrict__ C, const float *__restrict__ A, const float *__restrict__ W,
+                     int M, int N, int K, int lda, int ldc, size_t plane_stride) {
+    cd_gemm_tile<CG_BM>(C, A, W, M, N, K, lda, ldc, plane_stride);
+}
+
+/* The same product on 64 x 128 tiles (a wave owns 32 x 64): for row counts that 128-row tiles fit badly
+ * (1600 rows are 25 tiles of 64 but 12.5 of 128) and for launches whose 128-row tiles leave the last
+ * round of workgroups half empty. */
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, CG_W64)))
+vt_codec_gemm64_kernel(float *__restrict__ C, const float *__restrict__ A, const float *__restrict__ W,
+                       int M, int N, int K, int lda, int ldc, size_t plane_stride) {
+    cd_gemm_tile<64>(C, A, W, M, N, K, lda, ldc, plane_stride);
 }
 
 /* ---- row kernels ------------------------------------------------------------------------- */
@@ -539,19 +561,44 @@ static int cd_reserve(int n_frames) {
 }
 
 /* K is cut until the launch has about two workgroups per compute unit */
-static int cd_splits(int M, int N, int K) {
-    const int tiles = ((M + CG_BM - 1) / CG_BM) * ((N + CG_BN - 1) / CG_BN);
+static int cd_splits_bm(int M, int N, int K, int bm) {
+    const int tiles = ((M + bm - 1) / bm) * ((N + CG_BN - 1) / CG_BN);
     int s = 1;
     while (s < CD_MAX_SPLIT && tiles * s < 2 * g_vt.n_cu && (K / (s * 2)) % CG_BK == 0 && K / (s * 2) >= 128) s *= 2;
     return s;
 }
 
+/* Tile height and K cuts of a product: of the two tile heights the one whose busiest compute unit has
+ * less to do (workgroups per CU, rounded up, times the work of one), fewer cuts on a tie (their planes
+ * are written and read again), then the taller tile. */
+struct cd_plan { int bm, splits; };
+static cd_plan cd_plan_for(int M, int N, int K, int max_splits) {
+    cd_plan best = {CG_BM, 1};
+    long best_cost = -1;
+    const int heights[2] = {CG_BM, 64};
+    for (int h = 0; h < 2; h++) {
+        const int bm = heights[h];
+        int s = cd_splits_bm(M, N, K, bm);
+        while (s > max_splits) s /= 2;
+        const long wgs = (long)((M + bm - 1) / bm) * ((N + CG_BN - 1) / CG_BN) * s;
+        const long cost = ((wgs + g_vt.n_cu - 1) / g_vt.n_cu) * bm * (K / s);
+        if (best_cost < 0 || cost < best_cost || (cost == best_cost && s < best.splits)) {
+            best = cd_plan{bm, s};
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
 /* C planes (returns the number of planes written at stride M * ldc) */
-static int cd_gemm(float *C, const float *A, const float *W, int M, int N, int K, int lda, int ldc, int splits) {
-    dim3 grid((N + CG_BN - 1) / CG_BN, (M + CG_BM - 1) / CG_BM, splits);
-    hipLaunchKernelGGL(vt_codec_gemm_kernel, grid, dim3(256), 0, g_vt.stream, C, A, W, M, N, K, lda, ldc,
-                       (size_t)M * ldc);
-    return splits;
+static int cd_gemm(float *C, const float *A, const float *W, int M, int N, int K, int lda, int ldc, int max_splits = CD_MAX_SPLIT) {
+    const cd_plan pl = cd_plan_for(M, N, K, max_splits);
+    dim3 grid((N + CG_BN - 1) / CG_BN, (M + pl.bm - 1) / pl.bm, pl.splits);
+    if (pl.bm == CG_BM)
+        hipLaunchKernelGGL(vt_codec_gemm_kernel, grid, dim3(256), 0, g_vt.stream, C, A, W, M, N, K, lda, ldc, (size_t)M * ldc);
+    else
+        hipLaunchKernelGGL(vt_codec_gemm64_kernel, grid, dim3(256), 0, g_vt.stream, C, A, W, M, N, K, lda, ldc, (size_t)M * ldc);
+    return pl.splits;
 }
 
 static void cd_row(float *x_out, float *xn_out, const float *x_in, const float *planes, int splits, size_t plane_stride,
@@ -565,34 +612,38 @@ static int cd_enqueue(const int *d_codes, int n_frames, float *d_samples) {
     int T = n_frames;
     const float scale = 1.0f / sqrtf((float)CD_HEAD_DIM);
     hipLaunchKernelGGL(vt_codec_embed_kernel, dim3(T), dim3(256), 0, g_vt.stream, g_cd.wide, d_codes, g_cd.sem, T);
-    int sp = cd_gemm(g_cd.part, g_cd.wide, g_cd.w_in, T, CD_DIM, CD_IN_K, CD_IN_K, CD_DIM, cd_splits(T, CD_DIM, CD_IN_K));
+    int sp = cd_gemm(g_cd.part, g_cd.wide, g_cd.w_in, T, CD_DIM, CD_IN_K, CD_IN_K, CD_DIM);
     cd_row(g_cd.x, g_cd.xn, NULL, g_cd.part, sp, (size_t)T * CD_DIM, CD_DIM, g_cd.b_in, NULL,
            g_cd.layers[0].attention_norm, T);
     for (int li = 0; li < CD_LAYERS; li++) {
         const cd_layer_dev *l = &g_cd.layers[li];
-        sp = cd_gemm(g_cd.part, g_cd.xn, l->wqkv, T, 3 * CD_DIM, CD_DIM, CD_DIM, 3 * CD_DIM, cd_splits(T, 3 * CD_DIM, CD_DIM));
+        sp = cd_gemm(g_cd.part, g_cd.xn, l->wqkv, T, 3 * CD_DIM, CD_DIM, CD_DIM, 3 * CD_DIM);
         hipLaunchKernelGGL(vt_codec_qkv_kernel, dim3(T), dim3(256), 0, g_vt.stream, g_cd.qkv, g_cd.part, sp,
                            (size_t)T * 3 * CD_DIM, l->q_norm, l->k_norm);
         hipLaunchKernelGGL(vt_codec_attention_kernel, dim3((T * CD_HEADS + 3) / 4), dim3(256), 0, g_vt.stream,
                            g_cd.att, g_cd.qkv, T, l->window, g_cd.slopes, scale);
-        sp = cd_gemm(g_cd.part, g_cd.att, l->wo, T, CD_DIM, CD_DIM, CD_DIM, CD_DIM, cd_splits(T, CD_DIM, CD_DIM));
+        sp = cd_gemm(g_cd.part, g_cd.att, l->wo, T, CD_DIM, CD_DIM, CD_DIM, CD_DIM);
         cd_row(g_cd.x, g_cd.xn, g_cd.x, g_cd.part, sp, (size_t)T * CD_DIM, CD_DIM, NULL, l->attn_scale, l->ffn_norm, T);
-        sp = cd_gemm(g_cd.wide, g_cd.xn, l->w13, T, 2 * CD_HID, CD_DIM, CD_DIM, 2 * CD_HID, 1);
+        /* gate|up: uncut while its tiles fill the chip; the short stages (2 or 4 row tiles x 64) are cut
+         * in K like the other products and the SiLU x up pass sums the planes */
+        const int gu_tiles = ((T + CG_BM - 1) / CG_BM) * (2 * CD_HID / CG_BN);
+        int gu_cuts = gu_tiles <= g_vt.n_cu ? CD_MAX_SPLIT : 1;
+        while (gu_cuts > 1 && (size_t)T * gu_cuts > (size_t)g_cd.cap_frames * 8) gu_cuts /= 2;   /* the planes share the work area of the last stage's [8 n, 8192] */
+        sp = cd_gemm(g_cd.wide, g_cd.xn, l->w13, T, 2 * CD_HID, CD_DIM, CD_DIM, 2 * CD_HID, gu_cuts);
         {
             const size_t n = (size_t)T * CD_HID;
             const int blocks = (int)((n + 255) / 256 > 4096 ? 4096 : (n + 255) / 256);
-            hipLaunchKernelGGL(vt_codec_swiglu_kernel, dim3(blocks), dim3(256), 0, g_vt.stream, g_cd.h, g_cd.wide, 1,
-                               (size_t)0, n);
+            hipLaunchKernelGGL(vt_codec_swiglu_kernel, dim3(blocks), dim3(256), 0, g_vt.stream, g_cd.h, g_cd.wide, sp,
+                               (size_t)T * 2 * CD_HID, n);
         }
-        sp = cd_gemm(g_cd.part, g_cd.h, l->w2, T, CD_DIM, CD_HID, CD_HID, CD_DIM, cd_splits(T, CD_DIM, CD_HID));
+        sp = cd_gemm(g_cd.part, g_cd.h, l->w2, T, CD_DIM, CD_HID, CD_HID, CD_DIM);
         const int last_of_stage = (li & 1) == 1;
         const float *next_norm = (!last_of_stage) ? g_cd.layers[li + 1].attention_norm : NULL;
         cd_row(g_cd.x, g_cd.xn, g_cd.x, g_cd.part, sp, (size_t)T * CD_DIM, CD_DIM, NULL, l->ffn_scale, next_norm, T);
         if (last_of_stage && li < CD_LAYERS - 1) {
             const int st = li / 2;
             hipLaunchKernelGGL(vt_codec_pair_kernel, dim3(T), dim3(256), 0, g_vt.stream, g_cd.wide, g_cd.x, T);
-            sp = cd_gemm(g_cd.part, g_cd.wide, g_cd.w_up[st], T, 2 * CD_DIM, 2 * CD_DIM, 2 * CD_DIM, 2 * CD_DIM,
-                         cd_splits(T, 2 * CD_DIM, 2 * CD_DIM));
+            sp = cd_gemm(g_cd.part, g_cd.wide, g_cd.w_up[st], T, 2 * CD_DIM, 2 * CD_DIM, 2 * CD_DIM, 2 * CD_DIM);
             /* [T, 2048] planes are [2T, 1024] rows */
             cd_row(g_cd.x, g_cd.xn, NULL, g_cd.part, sp, (size_t)T * 2 * CD_DIM, CD_DIM, g_cd.b_up[st], NULL,
                    g_cd.layers[li + 1].attention_norm, 2 * T);
@@ -600,7 +651,7 @@ static int cd_enqueue(const int *d_codes, int n_frames, float *d_samples) {
         }
     }
     hipLaunchKernelGGL(vt_codec_taps_kernel, dim3(T), dim3(256), 0, g_vt.stream, g_cd.wide, g_cd.x, T, CD_OUT_TAPS);
-    sp = cd_gemm(g_cd.part, g_cd.wide, g_cd.w_out, T, CD_PATCH, CD_OUT_K, CD_OUT_K, CD_OUT_N, cd_splits(T, CD_OUT_N, CD_OUT_K));
+    sp = cd_gemm(g_cd.part, g_cd.wide, g_cd.w_out, T, CD_PATCH, CD_OUT_K, CD_OUT_K, CD_OUT_N);
     hipLaunchKernelGGL(vt_codec_wave_kernel, dim3(T), dim3(256), 0, g_vt.stream, d_samples, g_cd.part, sp,
                        (size_t)T * CD_OUT_N, CD_OUT_N, g_cd.b_out, T);
     return vt_check(hipGetLastError(), "codec launch");
@@ -662,7 +713,6 @@ int vt_codec_probe_launch(int which) {
     static const int NN[4] = {3 * CD_DIM, CD_DIM, 2 * CD_HID, CD_DIM}, KK[4] = {CD_DIM, CD_DIM, CD_DIM, CD_HID};
     if (which == 4) return cd_enqueue(g_cd.codes, frames, g_cd.wave);
     if (which < 0 || which > 3) return -1;
-    cd_gemm(Cc[which], A[which], W[which], T, NN[which], KK[which], KK[which], NN[which],
-            which == 2 ? 1 : cd_splits(T, NN[which], KK[which]));
+    cd_gemm(Cc[which], A[which], W[which], T, NN[which], KK[which], KK[which], NN[which], which == 2 ? 1 : CD_MAX_SPLIT);
     return 0;
 }
