@@ -102,6 +102,67 @@ def measured_traffic(workload):
         return None
 
 
+def live_decode_traffic(budget_s=150.0):
+    """HBM bytes per launch of the whole-step kernel, measured now: two child runs of this command under
+    rocprofv3 --pmc (FETCH_SIZE, then WRITE_SIZE; one counter per run), each with one launch of a plain
+    elementwise kernel of known traffic (--calibrate) that scales the counter.  Runs before this process
+    touches the GPU.  Returns (bytes, description) or (None, reason); never raises."""
+    import csv
+    import glob
+    import shutil
+    import signal
+    import subprocess
+    import tempfile
+    rocprof = shutil.which("rocprofv3") or "/opt/rocm/bin/rocprofv3"
+    if not os.path.exists(rocprof):
+        return None, "rocprofv3 not found"
+    steps, warmup = 6, 2
+    known_kib = {"FETCH_SIZE": 524288.0, "WRITE_SIZE": 262144.0}      # vt_add_kernel over 64 Mi floats
+    kib = {}
+    try:
+        out = tempfile.mkdtemp(prefix="vt_traffic_", dir="/tmp")
+    except OSError as e:
+        return None, "no scratch directory: %s" % e
+    try:
+        for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+            cmd = [rocprof, "--pmc", counter, "--output-format", "csv", "-d", os.path.join(out, counter), "-o", "t", "--",
+                   sys.executable, os.path.abspath(__file__), "--steps", str(steps), "--warmup", str(warmup),
+                   "--cpu-seconds", "0", "--calibrate", "--no-workloads", "--no-traffic"]
+            p = subprocess.Popen(cmd, cwd="/tmp", env=dict(os.environ, TMPDIR="/tmp"), stdout=subprocess.DEVNULL,
+                                 stderr=subprocess.DEVNULL, start_new_session=True)
+            try:
+                rc = p.wait(timeout=budget_s / 2)
+            except subprocess.TimeoutExpired:
+                os.killpg(p.pid, signal.SIGKILL)          # the process group this call started, nothing else
+                p.wait()
+                return None, "rocprofv3 --pmc %s did not finish in %.0f s" % (counter, budget_s / 2)
+            if rc != 0:
+                return None, "rocprofv3 --pmc %s exited with %d" % (counter, rc)
+            step, add = [], []
+            for path in glob.glob(os.path.join(out, counter, "**", "*counter_collection.csv"), recursive=True):
+                with open(path, newline="") as f:
+                    for row in csv.DictReader(f):
+                        if row.get("Counter_Name") != counter:
+                            continue
+                        name = row.get("Kernel_Name", "")
+                        if name.startswith("vt_decode_step_kernel"):
+                            step.append(float(row["Counter_Value"]))
+                        elif name.startswith("vt_add_kernel"):
+                            add.append(float(row["Counter_Value"]))
+            if not step or not add or min(add) <= 0:
+                return None, "no %s rows for the step kernel and the calibration kernel" % counter
+            kib[counter] = (sum(step) / len(step), known_kib[counter] / (sum(add) / len(add)), len(step))
+    except (OSError, ValueError, KeyError) as e:
+        return None, "traffic measurement failed: %s" % e
+    finally:
+        shutil.rmtree(out, ignore_errors=True)
+    (fk, ff, n), (wk, wf, _) = kib["FETCH_SIZE"], kib["WRITE_SIZE"]
+    desc = ("measured by this run: two child runs of this command under rocprofv3 --pmc (FETCH_SIZE %.1f KiB x %.3f, "
+            "WRITE_SIZE %.1f KiB x %.3f per launch, mean of %d launches at positions %d..%d; factors from a kernel of "
+            "known traffic in the same runs)" % (fk, ff, wk, wf, n, PROMPT, PROMPT + 2 * (warmup + steps)))
+    return 1024.0 * (fk * ff + wk * wf), desc
+
+
 TRAFFIC_SOURCE = "profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command, scaled by a copy kernel; not measured by this run)"
 
 
@@ -1011,6 +1072,9 @@ def main():
                     help="also launch one plain elementwise kernel (vt_add_kernel, a += b over 64 Mi floats: "
                          "512 MiB read, 256 MiB written) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "can be scaled by a kernel of known traffic")
+    ap.add_argument("--no-traffic", action="store_true",
+                    help="do not measure the step kernel's HBM traffic with two rocprofv3 --pmc child runs "
+                         "(roofline.traffic then comes from profiles/hbm_traffic.json)")
     ap.add_argument("--traffic-kib", type=float, default=None,
                     help="HBM bytes per launch measured with rocprofv3 --pmc (KiB), if known")
     args = ap.parse_args()
@@ -1031,6 +1095,13 @@ def main():
         return bench_layer(args)
     K, W = args.steps, args.warmup
     workers = min(16, os.cpu_count() or 8)
+
+    # HBM traffic of the step kernel, before this process touches the GPU (not under a profiler: a run
+    # that calibrates is one of the child runs itself, or somebody's own rocprofv3 command)
+    live_traffic, live_source = None, None
+    under_profiler = any(k.startswith("ROCP") for k in os.environ)
+    if args.mode == 0 and args.traffic_kib is None and not (args.no_traffic or args.calibrate or under_profiler):
+        live_traffic, live_source = live_decode_traffic()
 
     t0 = time.time()
     layers = make_layers(N_LAYERS, workers)
@@ -1137,7 +1208,15 @@ def main():
     avg_pos = pos0 + (K - 1) / 2.0
     bytes_launch = step_bytes(avg_pos)
     achieved = bytes_launch / (ms_kernel * 1e-3) / 1e9
-    traffic = measured_traffic("decode") if args.traffic_kib is None else args.traffic_kib * 1024.0
+    traffic_source = TRAFFIC_SOURCE
+    if args.traffic_kib is not None:
+        traffic, traffic_source = args.traffic_kib * 1024.0, "--traffic-kib"
+    elif live_traffic is not None:
+        traffic, traffic_source = live_traffic, live_source
+    else:
+        traffic = measured_traffic("decode")
+        if live_source:
+            traffic_source += "; live measurement skipped: " + live_source
     out = {
         "metric": "backbone decode ms/frame",
         "value": round(ms_step, 4),
@@ -1167,7 +1246,7 @@ def main():
             "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
-            "traffic_source": TRAFFIC_SOURCE if args.traffic_kib is None else "--traffic-kib",
+            "traffic_source": traffic_source,
             "bytes_per_launch": int(bytes_launch),
             "ms_per_launch": round(ms_kernel, 4),
             "stream_ceiling_gbps": round(nbytes_c.value / ms_ceiling / 1e6, 1),
